@@ -1,0 +1,177 @@
+/*
+ * t5attn.h -- C ABI of the MI355X (gfx950) T5 attention forward library.
+ *
+ * One shared library, libt5attn.so, replaces the Triton kernels behind the
+ * reference's attention hot path.  The reference has no FFI: its boundary is
+ * a set of Python functions that launch Triton kernels; each entry point below
+ * names the reference interface it stands in for (paths relative to the
+ * reference checkout).
+ *
+ * Conventions
+ *  - All tensor pointers are DEVICE pointers owned by the caller.  The library
+ *    never allocates, frees or retains device memory, and never synchronises
+ *    the host: every launch goes to the hipStream_t passed in (0 = null stream).
+ *  - Strides are in ELEMENTS.  The innermost (head_dim) stride must be 1, all
+ *    other strides multiples of 8 elements and base pointers 16-byte aligned.
+ *  - head_dim D is one of 16, 32, 64, 128 (reference: src/turbot5/ops/
+ *    fused_bias_attention.py:827-828).
+ *  - Every function returns T5A_OK (0) or a negative t5a_status; the message
+ *    of the last failure on the calling thread is t5a_last_error().
+ *  - Scores are q.k * sm_scale + bias; the T5 modules pass sm_scale = 1.0.
+ *  - The relative-position bias is never materialised: kernels derive
+ *    bucket(key_pos - query_pos) from integer positions and read the
+ *    (num_buckets, H) table.  Bucket boundaries are computed on the host with
+ *    the reference's fp32 formula (src/turbot5/model/attentions.py:78-124).
+ */
+#ifndef T5ATTN_H
+#define T5ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* t5a_stream_t; /* hipStream_t */
+
+typedef enum t5a_status {
+    T5A_OK = 0,
+    T5A_ERR_NULL = -1,      /* required pointer is NULL */
+    T5A_ERR_DTYPE = -2,     /* unsupported element type */
+    T5A_ERR_HEAD_DIM = -3,  /* D not in {16,32,64,128} */
+    T5A_ERR_SHAPE = -4,     /* negative or inconsistent sizes */
+    T5A_ERR_STRIDE = -5,    /* stride not a multiple of 8 elements / pointer not 16-byte aligned */
+    T5A_ERR_BUCKETS = -6,   /* num_buckets / max_distance outside the supported range */
+    T5A_ERR_PATTERN = -7,   /* unknown sparse pattern or bad pattern parameters */
+    T5A_ERR_WORKSPACE = -8, /* workspace missing or too small */
+    T5A_ERR_LAUNCH = -9     /* HIP reported an error at launch */
+} t5a_status;
+
+typedef enum t5a_dtype { T5A_BF16 = 0, T5A_F32 = 1, T5A_F16 = 2 } t5a_dtype;
+
+typedef enum t5a_pattern {
+    T5A_PATTERN_LOCAL = 1,   /* sliding window, |j-i| < block_len */
+    T5A_PATTERN_BLOCK = 2,   /* own block + first n_global tokens; the first n_global queries see everything */
+    T5A_PATTERN_TGLOBAL = 3  /* sliding window + side tokens (one per aux block of tokens) */
+} t5a_pattern;
+
+/* The (num_buckets, H) relative-attention table (nn.Embedding weight).  table == NULL: no bias. */
+typedef struct t5a_bias {
+    const void* table;
+    int32_t table_dtype;          /* T5A_F32, T5A_BF16 or T5A_F16 */
+    int32_t num_buckets;
+    int32_t max_distance;
+    int32_t reserved;
+    int64_t stride_bucket;        /* elements between buckets (torch stride(0)) */
+    int64_t stride_head;          /* elements between heads   (torch stride(1)) */
+} t5a_bias;
+
+int t5a_version(void);
+const char* t5a_last_error(void);
+
+/*
+ * Host-only, integer: bucket index for every relative position in
+ * [-max_distance, +max_distance] (out[rel + max_distance]); positions beyond
+ * that range share the bucket of the nearest end.  Replaces
+ * T5Attention._relative_position_bucket (src/turbot5/model/attentions.py:78-124).
+ */
+int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t* out /* 2*max_distance+1 */);
+
+/*
+ * Dense fused-bias flash attention forward.
+ * Replaces flash_attention_with_fusing_bias / flash_attn_v2_fwd_bias
+ * (src/turbot5/ops/fused_bias_attention.py:876-890, :23-59).
+ * q,o: (B,H,M,D); k,v: (B,H,N,D); strides = {batch, head, row}.
+ * Queries are aligned to the end of the keys: rel = j - (i + N - M); with
+ * causal != 0 key j is visible iff j <= i + N - M and buckets are
+ * unidirectional, else bidirectional.  lse (optional) is (B,H,M) contiguous
+ * fp32, natural log of the softmax normaliser (fused_bias_attention.py:358).
+ */
+typedef struct t5a_dense_args {
+    const void* q; const void* k; const void* v; void* o; float* lse;
+    int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
+    int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
+    int32_t causal; float sm_scale;
+    t5a_bias bias;
+} t5a_dense_args;
+int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
+
+/*
+ * Packed variable-length forward.
+ * Replaces flash_attention_with_fusing_bias_varlen / flash_attn_v2_fwd_bias
+ * (src/turbot5/ops/varlen_fused_bias_attn.py:870-889, :37-80); the q-tile work
+ * list of get_mid (:23-35) is derived on the device from cu_seqlens, so there
+ * is no host synchronisation.
+ * q,o: (total_q,H,D); k,v: (total_k,H,D); strides = {row, head}.
+ * cu_seqlens_q/k: DEVICE int32 arrays of B+1 ascending offsets.  Positions are
+ * in-sequence; per sequence the semantics equal t5a_fwd_dense.
+ * lse (optional) is (total_q,H) contiguous fp32.
+ */
+typedef struct t5a_varlen_args {
+    const void* q; const void* k; const void* v; void* o; float* lse;
+    int64_t q_strides[2]; int64_t k_strides[2]; int64_t v_strides[2]; int64_t o_strides[2];
+    const int32_t* cu_seqlens_q; const int32_t* cu_seqlens_k;
+    int32_t dtype; int32_t B; int32_t H; int32_t D;
+    int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
+    int32_t causal; float sm_scale;
+    t5a_bias bias;
+} t5a_varlen_args;
+int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
+
+/*
+ * Sparse encoder self-attention as tile skipping (no bias/mask tensor, no
+ * replicated K/V).  Replaces the blocked torch code + flash_attention_with_bias
+ * (src/turbot5/ops/flash_attention.py:870-884) in T5LocalAttention.forward
+ * (src/turbot5/model/attentions.py:583-638), T5BlockAttention.forward (:788-853)
+ * and T5TransientGlobalAttention.forward (:977-1052), all-ones attention mask.
+ * q,k,v,o: (B,H,L,D); strides = {batch, head, row}.
+ *   LOCAL   block_len = window; keys |j-i| < block_len, bias bucket(j-i).
+ *   BLOCK   block_len, aux = number of global tokens G (G <= block_len).
+ *           Rows < G: all keys.  Other rows: the G global tokens with
+ *           rel = g-(G+i%block_len) and the own block with rel = j-i; in block 0
+ *           only the first block_len-G own-block tokens are visible and keys of
+ *           a ragged last block past L count as zero vectors (both as the
+ *           reference computes them, attentions.py:722-732, :807-814).
+ *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
+ *           (B,H,n_side,D) projected block aggregates, bias bucket(g - i/aux).
+ */
+typedef struct t5a_sparse_args {
+    const void* q; const void* k; const void* v; void* o;
+    const void* side_k; const void* side_v;
+    int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
+    int64_t side_k_strides[3]; int64_t side_v_strides[3];
+    int32_t dtype; int32_t B; int32_t H; int32_t L; int32_t D;
+    int32_t pattern; int32_t block_len; int32_t aux; int32_t n_side;
+    float sm_scale; int32_t reserved;
+    t5a_bias bias;
+} t5a_sparse_args;
+int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);
+
+/*
+ * Flash-decoding split-K forward for few query rows over a long memory.
+ * Replaces flash_attn_v2_fwd (src/turbot5/ops/flash_decoding.py:6-55): the
+ * per-split kernel (:57-178) and the merge the reference does in torch (:47-55).
+ * q,o: (B,H,M,D), M <= 16; k,v: (B,H,N,D); strides = {batch, head, row}.
+ * attn_bias (optional): additive fp32 bias, strides {batch, head, row, col},
+ * use 0 to broadcast.  Split s covers keys [s*(N/S), (s+1)*(N/S)), the last
+ * split also the remainder.  workspace holds, contiguous fp32, in this order:
+ * part_o (B,H,S,M,D) normalised partial outputs, part_l (B,H,S,M) partial
+ * sums of exp, part_m (B,H,S,M) partial maxima (scaled scores, natural units).
+ */
+typedef struct t5a_splitk_args {
+    const void* q; const void* k; const void* v; void* o;
+    const float* attn_bias;
+    void* workspace; int64_t workspace_bytes;
+    int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
+    int64_t bias_strides[4];
+    int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
+    int32_t num_splits; float sm_scale;
+} t5a_splitk_args;
+int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, int32_t num_splits);
+int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* T5ATTN_H */

@@ -1,0 +1,157 @@
+"""GPU parity of the dense and packed fused-bias forwards against the CPU oracle.
+
+Tolerances (max-abs): bf16/fp16 2e-2, fp32 1e-4 -- the bars the build was given.
+The oracle runs fp32 math on the same (already rounded) inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import t5_basic as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 2e-2, torch.float32: 1e-4}
+
+
+def rnd(*shape, seed=0, scale=0.5, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(*shape, generator=g)).to(dtype)
+
+
+def run_dense(dev, B, H, M, N, D, dtype, causal, bias=True, sm_scale=1.0, seed=0, nb=32, md=128, blhd=False):
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    if blhd:   # (B,H,L,D) views of (B,L,H,D) memory, as the attention modules produce them
+        q = rnd(B, M, H, D, seed=seed, dtype=dtype).transpose(1, 2)
+        k = rnd(B, N, H, D, seed=seed + 1, dtype=dtype).transpose(1, 2)
+        v = rnd(B, N, H, D, seed=seed + 2, dtype=dtype).transpose(1, 2)
+    else:
+        q, k, v = (rnd(B, H, L, D, seed=seed + i, dtype=dtype) for i, L in enumerate((M, N, N)))
+    table = rnd(nb, H, seed=seed + 3, scale=1.0) if bias else None
+    out, lse = flash_attention_with_fusing_bias(q.to(dev), k.to(dev), v.to(dev), None if table is None else table.to(dev),
+                                                causal=causal, sm_scale=sm_scale, NUM_BUCKETS=nb, MAX_DISTANCE=md,
+                                                return_lse=True)
+    torch.cuda.synchronize()
+    assert out.shape == q.shape and out.dtype == dtype
+    want = O.dense_attention(q, k, v, table, causal, sm_scale, nb, md)
+    err = (out.float().cpu() - want).abs().max().item()
+    want_lse = O.dense_lse(q, k, table, causal, sm_scale, nb, md)
+    fin = torch.isfinite(want_lse)
+    lse_err = (lse.cpu()[fin] - want_lse[fin]).abs().max().item() if fin.any() else 0.0
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    return err, lse_err
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("M,N", [(128, 128), (256, 256), (100, 100), (1, 77), (77, 300), (300, 77), (513, 513)])
+def test_dense_bf16_shapes(gpu_device, causal, M, N):
+    err, lse_err = run_dense(gpu_device, 2, 3, M, N, 64, torch.bfloat16, causal)
+    assert err <= TOL[torch.bfloat16], err
+    assert lse_err <= 2e-2, lse_err
+
+
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_dense_head_dims_and_dtypes(gpu_device, D, dtype):
+    for causal in (False, True):
+        err, lse_err = run_dense(gpu_device, 1, 2, 200, 200, D, dtype, causal, seed=5)
+        assert err <= TOL[dtype], (err, causal)
+        assert lse_err <= (1e-3 if dtype == torch.float32 else 2e-2)
+
+
+def test_dense_strided_views(gpu_device):
+    err, _ = run_dense(gpu_device, 2, 4, 333, 333, 64, torch.bfloat16, False, blhd=True, seed=7)
+    assert err <= 2e-2
+    err, _ = run_dense(gpu_device, 2, 4, 200, 200, 64, torch.float32, True, blhd=True, seed=8)
+    assert err <= 1e-4
+
+
+def test_dense_no_bias_default_scale(gpu_device):
+    err, _ = run_dense(gpu_device, 1, 2, 150, 150, 64, torch.bfloat16, False, bias=False, sm_scale=None, seed=9)
+    assert err <= 2e-2
+
+
+def test_dense_other_bucket_params(gpu_device):
+    for nb, md in ((64, 256), (16, 64), (32, 20)):
+        err, _ = run_dense(gpu_device, 1, 2, 400, 400, 64, torch.float32, False, nb=nb, md=md, seed=10)
+        assert err <= 1e-4, (nb, md, err)
+
+
+def test_config2_shape_subset(gpu_device):
+    """BASELINE config 2 (B16 H12 L1024 D64 bf16, N(0,1)*0.5, table N(0,1)); oracle on 2 batches."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (0.5 * torch.randn(16, 12, 1024, 64, generator=g) for _ in range(3))
+    table = torch.randn(32, 12, generator=g)
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (q, k, v))
+    out = flash_attention_with_fusing_bias(qb.to(gpu_device), kb.to(gpu_device), vb.to(gpu_device),
+                                           table.to(gpu_device), causal=False, sm_scale=1.0)
+    for b in (0, 15):
+        want = O.dense_attention(qb[b:b + 1], kb[b:b + 1], vb[b:b + 1], table, False, 1.0)
+        assert (out[b:b + 1].float().cpu() - want).abs().max().item() <= 2e-2
+    # literal bf16 'basic' (scores and weights rounded to bf16) is further from fp32 truth than the kernel
+    lit = O.dense_attention(qb[:1], kb[:1], vb[:1], table, False, 1.0, compute_dtype=torch.bfloat16).float()
+    assert (out[:1].float().cpu() - lit).abs().max().item() <= 4e-2
+
+
+def test_long_sequence_properties(gpu_device):
+    """L = 8192: V = 1 gives exactly 1; a constant table shift changes nothing (size-independent checks)."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    B, H, Lq, D = 1, 4, 8192, 64
+    q = rnd(B, H, Lq, D, seed=11, dtype=torch.bfloat16).to(gpu_device)
+    k = rnd(B, H, Lq, D, seed=12, dtype=torch.bfloat16).to(gpu_device)
+    ones = torch.ones(B, H, Lq, D, dtype=torch.bfloat16, device=gpu_device)
+    table = rnd(32, H, seed=13, scale=1.0).to(gpu_device)
+    out = flash_attention_with_fusing_bias(q, k, ones, table, sm_scale=1.0)
+    assert (out.float() - 1.0).abs().max().item() <= 1e-2
+    v = rnd(B, H, Lq, D, seed=14, dtype=torch.bfloat16).to(gpu_device)
+    a = flash_attention_with_fusing_bias(q, k, v, table, sm_scale=1.0)
+    b = flash_attention_with_fusing_bias(q, k, v, table + 2.5, sm_scale=1.0)
+    assert (a.float() - b.float()).abs().max().item() <= 1e-2
+    # oracle on a random subset of 256 query rows of head 1
+    rows = torch.randperm(Lq, generator=torch.Generator().manual_seed(15))[:256].sort().values
+    qc, kc, vc = q.cpu()[:, 1:2], k.cpu()[:, 1:2], v.cpu()[:, 1:2]
+    tb = table.cpu()[:, 1:2]
+    i = rows[:, None]
+    j = torch.arange(Lq)[None, :]
+    bias = tb[O.relative_position_bucket(j - i, True, 32, 128)].permute(2, 0, 1).unsqueeze(0)
+    want = O.basic_attention(qc[:, :, rows].float(), kc.float(), vc.float(), bias)
+    assert (a[:, 1:2, rows].float().cpu() - want).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_varlen(gpu_device, causal, dtype):
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    H, D = 3, 64
+    lens = [5, 128, 0, 129, 300, 1, 64]
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    tot = int(cu[-1])
+    q, k, v = (rnd(tot, H, D, seed=20 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=23, scale=1.0)
+    out, lse = flash_attention_with_fusing_bias_varlen(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                                       table.to(gpu_device), cu.to(gpu_device), cu.to(gpu_device),
+                                                       max(lens), max(lens), causal=causal, sm_scale=1.0,
+                                                       return_lse=True)
+    want = O.varlen_attention(q, k, v, table, cu, cu, causal, 1.0)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
+    assert lse.shape == (tot, H) and torch.isfinite(lse).all()
+
+
+def test_varlen_cross_lengths(gpu_device):
+    """different q and k lengths per sequence (decoder step over a padded cache)."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    H, D = 2, 64
+    lq, lk = [1, 3, 130], [40, 200, 130]
+    cq = torch.tensor([0] + list(np.cumsum(lq)), dtype=torch.int32)
+    ck = torch.tensor([0] + list(np.cumsum(lk)), dtype=torch.int32)
+    q = rnd(int(cq[-1]), H, D, seed=30, dtype=torch.bfloat16)
+    k = rnd(int(ck[-1]), H, D, seed=31, dtype=torch.bfloat16)
+    v = rnd(int(ck[-1]), H, D, seed=32, dtype=torch.bfloat16)
+    table = rnd(32, H, seed=33, scale=1.0)
+    for causal in (False, True):
+        out = flash_attention_with_fusing_bias_varlen(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                                      table.to(gpu_device), cq.to(gpu_device), ck.to(gpu_device),
+                                                      max(lq), max(lk), causal=causal, sm_scale=1.0)
+        want = O.varlen_attention(q, k, v, table, cq, ck, causal, 1.0)
+        assert (out.float().cpu() - want).abs().max().item() <= 2e-2

@@ -1,0 +1,107 @@
+"""GPU parity of the local / block / transient-global forwards and the split-K decode kernel."""
+import pytest
+import torch
+
+from oracle import t5_basic as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 2e-2, torch.float32: 1e-4}
+
+
+def rnd(*shape, seed=0, scale=0.5, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(*shape, generator=g)).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl", [(512, 128), (256, 16), (384, 64), (1024, 512), (100, 128), (640, 128)])
+def test_local(gpu_device, dtype, L, Bl):
+    from turbot5_amd.ops import local_attention_with_fusing_bias
+    B, H, D = 2, 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=40 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=43, scale=1.0)
+    out = local_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                           table.to(gpu_device), Bl)
+    want = O.local_attention_blocked(q, k, v, table, Bl)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
+
+
+def test_local_ragged_length_matches_closed_form(gpu_device):
+    """L not a multiple of block_len: the reference's blocked code cannot run; the window definition can."""
+    from turbot5_amd.ops import local_attention_with_fusing_bias
+    B, H, L, D, Bl = 1, 2, 333, 64, 100
+    q, k, v = (rnd(B, H, L, D, seed=50 + i) for i in range(3))
+    table = rnd(32, H, seed=53, scale=1.0)
+    out = local_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                           table.to(gpu_device), Bl)
+    i = torch.arange(L)[:, None]
+    j = torch.arange(L)[None, :]
+    bias = table[O.relative_position_bucket(j - i, True, 32, 128)].permute(2, 0, 1).unsqueeze(0)
+    bias = bias.masked_fill((j - i).abs() >= Bl, float("-inf"))
+    want = O.basic_attention(q, k, v, bias)
+    assert (out.cpu() - want).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,G", [(512, 128, 64), (256, 32, 8), (384, 128, 128), (300, 128, 64), (100, 128, 64),
+                                    (1024, 512, 32), (256, 64, 0)])
+def test_block(gpu_device, dtype, L, Bl, G):
+    from turbot5_amd.ops import block_attention_with_fusing_bias
+    B, H, D = 2, 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=60 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=63, scale=1.0)
+    out = block_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                           table.to(gpu_device), Bl, G)
+    want = O.block_attention_blocked(q, k, v, table, Bl, G)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,gbs", [(512, 128, 16), (256, 32, 8), (2048, 128, 16), (384, 64, 1)])
+def test_tglobal(gpu_device, dtype, L, Bl, gbs):
+    from turbot5_amd.ops import transient_global_attention_with_fusing_bias
+    B, H, D = 2, 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=70 + i, dtype=dtype) for i in range(3))
+    sk, sv = (rnd(B, H, L // gbs, D, seed=73 + i, dtype=dtype) for i in range(2))
+    table = rnd(32, H, seed=75, scale=1.0)
+    out = transient_global_attention_with_fusing_bias(*(t.to(gpu_device) for t in (q, k, v, sk, sv)),
+                                                      table.to(gpu_device), Bl, gbs)
+    want = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs)
+    assert (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,S", [(1, 1000, 4), (1, 8192, 8), (3, 500, 7), (8, 257, 2), (1, 5, 8), (1, 300, None)])
+def test_splitk(gpu_device, dtype, M, N, S):
+    from turbot5_amd.ops import flash_attn_v2_fwd, flash_decoding_attention
+    B, H, D = 3, 4, 64
+    # (B,H,N,D) views of a (B,N,H,D) cache, as the decoder keeps it
+    q = rnd(B, H, M, D, seed=80, dtype=dtype)
+    k = rnd(B, N, H, D, seed=81, dtype=dtype).transpose(1, 2)
+    v = rnd(B, N, H, D, seed=82, dtype=dtype).transpose(1, 2)
+    res, Lsum, ml = flash_attn_v2_fwd(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None, False, 1.0, S)
+    want = O.dense_attention(q, k, v, None, False, 1.0)
+    assert res.dtype == torch.float32
+    assert (res.cpu() - want).abs().max().item() <= TOL[dtype]
+    if S is not None:
+        so, l, m = O.splitk_partials(q, k, v, S, 1.0)
+        l_, m_ = (l.squeeze(-1), m.squeeze(-1)) if M == 1 else (l, m)
+        live = l_ > 0
+        assert (ml.cpu()[live] - m_[live]).abs().max().item() <= 2e-2
+        assert ((Lsum.cpu()[live] - l_[live]).abs() / l_[live]).max().item() <= 2e-2
+    out = flash_decoding_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None, 1.0, S)
+    assert out.dtype == dtype and (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
+
+
+def test_splitk_with_bias_and_head_dims(gpu_device):
+    from turbot5_amd.ops import flash_attn_v2_fwd
+    for D in (16, 32, 128):
+        B, H, M, N = 2, 2, 2, 333
+        q, k, v = rnd(B, H, M, D, seed=90), rnd(B, H, N, D, seed=91), rnd(B, H, N, D, seed=92)
+        bias = rnd(1, H, M, N, seed=93, scale=1.0)
+        res, _, _ = flash_attn_v2_fwd(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), bias.to(gpu_device),
+                                      False, 0.8, 3)
+        s = torch.einsum("bhqd,bhkd->bhqk", q * 0.8, k) + bias
+        want = torch.softmax(s, -1) @ v
+        assert (res.cpu() - want).abs().max().item() <= 1e-4

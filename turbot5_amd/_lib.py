@@ -1,0 +1,117 @@
+"""ctypes binding of libt5attn.so (the C ABI declared in include/t5attn.h).
+
+There is no fallback: if the library is missing or a call fails, an exception
+is raised.  Build the library with ``python -m turbot5_amd.build``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libt5attn.so")
+
+T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
+PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
+
+EXPORTS = (
+    "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
+    "t5a_fwd_sparse", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk",
+)
+
+
+class T5ABias(C.Structure):
+    _fields_ = [("table", C.c_void_p), ("table_dtype", C.c_int32), ("num_buckets", C.c_int32),
+                ("max_distance", C.c_int32), ("reserved", C.c_int32),
+                ("stride_bucket", C.c_int64), ("stride_head", C.c_int64)]
+
+
+class T5ADenseArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
+                ("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3),
+                ("o_strides", C.c_int64 * 3),
+                ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("M", C.c_int32), ("N", C.c_int32),
+                ("D", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
+                ("bias", T5ABias)]
+
+
+class T5AVarlenArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
+                ("q_strides", C.c_int64 * 2), ("k_strides", C.c_int64 * 2), ("v_strides", C.c_int64 * 2),
+                ("o_strides", C.c_int64 * 2),
+                ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
+                ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
+                ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32),
+                ("max_seqlen_k", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
+                ("bias", T5ABias)]
+
+
+class T5ASparseArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+                ("side_k", C.c_void_p), ("side_v", C.c_void_p),
+                ("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3),
+                ("o_strides", C.c_int64 * 3), ("side_k_strides", C.c_int64 * 3), ("side_v_strides", C.c_int64 * 3),
+                ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("L", C.c_int32), ("D", C.c_int32),
+                ("pattern", C.c_int32), ("block_len", C.c_int32), ("aux", C.c_int32), ("n_side", C.c_int32),
+                ("sm_scale", C.c_float), ("reserved", C.c_int32),
+                ("bias", T5ABias)]
+
+
+class T5ASplitKArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+                ("attn_bias", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
+                ("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3),
+                ("o_strides", C.c_int64 * 3), ("bias_strides", C.c_int64 * 4),
+                ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("M", C.c_int32), ("N", C.c_int32),
+                ("D", C.c_int32), ("num_splits", C.c_int32), ("sm_scale", C.c_float)]
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+class T5AError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libt5attn error {code}: {message}")
+        self.code = code
+
+
+def load() -> C.CDLL:
+    """Load (once) and return the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: the HIP extension is not built (run `python -m turbot5_amd.build`); "
+                "there is no fallback path")
+        lib = C.CDLL(LIB_PATH)
+        lib.t5a_version.restype = C.c_int
+        lib.t5a_last_error.restype = C.c_char_p
+        lib.t5a_bucket_lut.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32)]
+        lib.t5a_bucket_lut.restype = C.c_int
+        for name, typ in (("t5a_fwd_dense", T5ADenseArgs), ("t5a_fwd_varlen", T5AVarlenArgs),
+                          ("t5a_fwd_sparse", T5ASparseArgs), ("t5a_fwd_splitk", T5ASplitKArgs)):
+            fn = getattr(lib, name)
+            fn.argtypes = [C.POINTER(typ), C.c_void_p]
+            fn.restype = C.c_int
+        lib.t5a_splitk_workspace_bytes.argtypes = [C.c_int32] * 5
+        lib.t5a_splitk_workspace_bytes.restype = C.c_int64
+        _lib = lib
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise T5AError(rc, load().t5a_last_error().decode("utf-8", "replace"))
+
+
+def bucket_lut(bidirectional: bool, num_buckets: int, max_distance: int):
+    """Host-side integer bucket table for rel in [-max_distance, max_distance] as a python list."""
+    out = (C.c_int32 * (2 * max_distance + 1))()
+    check(load().t5a_bucket_lut(int(bool(bidirectional)), num_buckets, max_distance, out))
+    return list(out)

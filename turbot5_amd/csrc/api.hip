@@ -1,0 +1,338 @@
+// extern "C" entry points of libt5attn.so: argument validation, bucket
+// boundaries on the host, parameter packing, launch.  See include/t5attn.h.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "t5a_internal.h"
+
+namespace t5a {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// Bucket of one relative position with the arithmetic of the reference
+// (src/turbot5/model/attentions.py:97-124): fp32 division, fp32 log, fp32
+// division by the double constant rounded to fp32, fp32 multiply, truncation.
+static int bucket_scalar(int rel, bool bidirectional, int num_buckets, int max_distance) {
+    int nb = num_buckets, out = 0, d;
+    if (bidirectional) {
+        nb /= 2;
+        if (rel > 0) out += nb;
+        d = rel < 0 ? -rel : rel;
+    } else {
+        d = rel < 0 ? -rel : 0;
+    }
+    const int max_exact = nb / 2;
+    if (d < max_exact) return out + d;
+    const float x = logf((float)d / (float)max_exact);
+    const float den = (float)log((double)max_distance / (double)max_exact);
+    const float y = x / den * (float)(nb - max_exact);
+    long big = (long)max_exact + (long)y;
+    if (big > nb - 1) big = nb - 1;
+    return out + (int)big;
+}
+
+static int check_bucket_params(bool bidirectional, int num_buckets, int max_distance) {
+    const int nb = bidirectional ? num_buckets / 2 : num_buckets;
+    const int max_exact = nb / 2;
+    if (num_buckets <= 0 || max_exact < 1 || nb > 2 * kMaxThresholds)
+        return fail(T5A_ERR_BUCKETS, "num_buckets=%d unsupported (need %d..%d)", num_buckets,
+                    bidirectional ? 4 : 2, bidirectional ? 4 * kMaxThresholds : 2 * kMaxThresholds);
+    if (max_distance <= max_exact)
+        return fail(T5A_ERR_BUCKETS, "max_distance=%d must exceed num_buckets/%d=%d", max_distance,
+                    bidirectional ? 4 : 2, max_exact);
+    return T5A_OK;
+}
+
+int make_bucket_spec(bool bidirectional, int num_buckets, int max_distance, BucketSpec* out) {
+    static std::mutex mu;
+    static std::map<std::tuple<int, int, int>, BucketSpec> cache;
+    const auto key = std::make_tuple((int)bidirectional, num_buckets, max_distance);
+    {
+        std::lock_guard<std::mutex> g(mu);
+        auto it = cache.find(key);
+        if (it != cache.end()) { *out = it->second; return T5A_OK; }
+    }
+    int rc = check_bucket_params(bidirectional, num_buckets, max_distance);
+    if (rc != T5A_OK) return rc;
+    BucketSpec s;
+    memset(&s, 0, sizeof(s));
+    s.bidirectional = bidirectional ? 1 : 0;
+    s.nb = bidirectional ? num_buckets / 2 : num_buckets;
+    s.max_exact = s.nb / 2;
+    s.n_thr = s.nb - 1 - s.max_exact;
+    // walk the distances once; the device code counts thresholds, which is exact
+    // only for a non-decreasing sequence of buckets
+    int prev = s.max_exact, filled = 0;
+    for (int d = s.max_exact; d <= max_distance; ++d) {
+        const int bk = bucket_scalar(-d, bidirectional, num_buckets, max_distance);
+        if (bk < prev) return fail(T5A_ERR_BUCKETS, "bucket sequence not monotone at distance %d", d);
+        while (filled < bk - s.max_exact && filled < s.n_thr) s.thr[filled++] = d;
+        prev = bk;
+    }
+    if (prev != s.nb - 1 || filled != s.n_thr)
+        return fail(T5A_ERR_BUCKETS, "buckets do not saturate at max_distance=%d", max_distance);
+    s.sat = s.n_thr > 0 ? s.thr[s.n_thr - 1] : s.max_exact;
+    if (s.sat > kMaxSaturation)
+        return fail(T5A_ERR_BUCKETS, "bucket saturation distance %d exceeds %d", s.sat, kMaxSaturation);
+    {
+        std::lock_guard<std::mutex> g(mu);
+        cache[key] = s;
+    }
+    *out = s;
+    return T5A_OK;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// unit: strides must be multiples of this many elements (16 bytes worth, or 1 for scalar stores)
+static int check_tensor(const char* name, const void* ptr, const int64_t* strides, int n, int unit) {
+    if (ptr == nullptr) return fail(T5A_ERR_NULL, "%s is NULL", name);
+    if (unit > 1 && !aligned16(ptr)) return fail(T5A_ERR_STRIDE, "%s is not 16-byte aligned", name);
+    for (int i = 0; i < n; ++i)
+        if (strides[i] % unit != 0)
+            return fail(T5A_ERR_STRIDE, "%s stride[%d]=%lld is not a multiple of %d elements", name, i, (long long)strides[i], unit);
+    return T5A_OK;
+}
+
+static int check_common(int dtype, int D) {
+    if (dtype != T5A_BF16 && dtype != T5A_F16 && dtype != T5A_F32) return fail(T5A_ERR_DTYPE, "unsupported dtype %d", dtype);
+    if (D != 16 && D != 32 && D != 64 && D != 128) return fail(T5A_ERR_HEAD_DIM, "head_dim %d not in {16,32,64,128}", D);
+    return T5A_OK;
+}
+
+static int fill_bias(const t5a_bias& b, bool bidirectional, FwdParams* p) {
+    p->table = b.table;
+    p->table_dtype = b.table_dtype;
+    p->t_sbucket = b.stride_bucket;
+    p->t_shead = b.stride_head;
+    memset(&p->bs, 0, sizeof(p->bs));
+    if (b.table == nullptr) return T5A_OK;
+    if (b.table_dtype != T5A_F32 && b.table_dtype != T5A_BF16 && b.table_dtype != T5A_F16)
+        return fail(T5A_ERR_DTYPE, "unsupported bias table dtype %d", b.table_dtype);
+    return make_bucket_spec(bidirectional, b.num_buckets, b.max_distance, &p->bs);
+}
+
+static int finish(hipError_t e, const char* what) {
+    if (e != hipSuccess) return fail(T5A_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return T5A_OK;
+}
+
+static const float kLog2e = 1.4426950408889634f;
+
+static hipError_t launch_fwd(const FwdParams& p, int dtype, int D, int mode, bool causal, hipStream_t stream) {
+    if (p.total_items <= 0) return hipSuccess;
+    if (dtype == T5A_BF16) return launch_fwd_bf16(p, D, mode, causal, stream);
+    if (dtype == T5A_F16) return launch_fwd_f16(p, D, mode, causal, stream);
+    if (dtype == T5A_F32) return launch_fwd_f32(p, D, mode, causal, stream);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace t5a
+
+using namespace t5a;
+
+extern "C" {
+
+int t5a_version(void) { return 100; }
+
+const char* t5a_last_error(void) { return g_err; }
+
+int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t* out) {
+    if (out == nullptr) return fail(T5A_ERR_NULL, "out is NULL");
+    int rc = check_bucket_params(bidirectional != 0, num_buckets, max_distance);
+    if (rc != T5A_OK) return rc;
+    for (int rel = -max_distance; rel <= max_distance; ++rel)
+        out[rel + max_distance] = bucket_scalar(rel, bidirectional != 0, num_buckets, max_distance);
+    return T5A_OK;
+}
+
+int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if (a->B < 0 || a->H <= 0 || a->M < 0 || a->N < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d M=%d N=%d", a->B, a->H, a->M, a->N);
+    if (a->B == 0 || a->M == 0) return T5A_OK;
+    if ((rc = check_tensor("q", a->q, a->q_strides, 3, unit))) return rc;
+    if ((rc = check_tensor("o", a->o, a->o_strides, 3, unit))) return rc;
+    if (a->N > 0) {
+        if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
+        if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
+    }
+    FwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
+    p.q_sb = a->q_strides[0]; p.q_sh = a->q_strides[1]; p.q_sr = a->q_strides[2];
+    p.k_sb = a->k_strides[0]; p.k_sh = a->k_strides[1]; p.k_sr = a->k_strides[2];
+    p.v_sb = a->v_strides[0]; p.v_sh = a->v_strides[1]; p.v_sr = a->v_strides[2];
+    p.o_sb = a->o_strides[0]; p.o_sh = a->o_strides[1]; p.o_sr = a->o_strides[2];
+    p.lse_sb = (int64_t)a->H * a->M; p.lse_sh = a->M; p.lse_sr = 1;
+    p.B = a->B; p.H = a->H; p.M = a->M; p.N = a->N;
+    p.align_end = 1;
+    p.tiles_per_seq = (a->M + 127) / 128;
+    const int64_t items = (int64_t)p.tiles_per_seq * a->H * a->B;
+    if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
+    p.total_items = (int)items;
+    p.c1 = a->sm_scale * kLog2e;
+    if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
+    return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
+}
+
+int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if (a->B < 0 || a->H <= 0 || a->total_q < 0 || a->total_k < 0)
+        return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d total_q=%d total_k=%d", a->B, a->H, a->total_q, a->total_k);
+    if (a->B == 0 || a->total_q == 0) return T5A_OK;
+    if (a->cu_seqlens_q == nullptr || a->cu_seqlens_k == nullptr) return fail(T5A_ERR_NULL, "cu_seqlens is NULL");
+    if ((rc = check_tensor("q", a->q, a->q_strides, 2, unit))) return rc;
+    if ((rc = check_tensor("o", a->o, a->o_strides, 2, unit))) return rc;
+    if (a->total_k > 0) {
+        if ((rc = check_tensor("k", a->k, a->k_strides, 2, unit))) return rc;
+        if ((rc = check_tensor("v", a->v, a->v_strides, 2, unit))) return rc;
+    }
+    FwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
+    p.q_sr = a->q_strides[0]; p.q_sh = a->q_strides[1];
+    p.k_sr = a->k_strides[0]; p.k_sh = a->k_strides[1];
+    p.v_sr = a->v_strides[0]; p.v_sh = a->v_strides[1];
+    p.o_sr = a->o_strides[0]; p.o_sh = a->o_strides[1];
+    p.lse_sr = a->H; p.lse_sh = 1;
+    p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+    p.B = a->B; p.H = a->H; p.M = a->max_seqlen_q; p.N = a->max_seqlen_k;
+    // sum_b ceil(len_b / 128) <= total_q / 128 + B: launch that many, the surplus exits
+    const int64_t items = ((int64_t)a->total_q / 128 + a->B) * a->H;
+    if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
+    p.total_items = (int)items;
+    p.tiles_per_seq = 1;
+    p.align_end = 1;
+    p.c1 = a->sm_scale * kLog2e;
+    if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
+    return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
+}
+
+int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if (a->B < 0 || a->H <= 0 || a->L < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d L=%d", a->B, a->H, a->L);
+    if (a->pattern != T5A_PATTERN_LOCAL && a->pattern != T5A_PATTERN_BLOCK && a->pattern != T5A_PATTERN_TGLOBAL)
+        return fail(T5A_ERR_PATTERN, "unknown pattern %d", a->pattern);
+    if (a->block_len <= 0) return fail(T5A_ERR_PATTERN, "block_len=%d must be positive", a->block_len);
+    if (a->pattern == T5A_PATTERN_BLOCK && (a->aux < 0 || a->aux > a->block_len))
+        return fail(T5A_ERR_PATTERN, "block pattern needs 0 <= n_global (%d) <= block_len (%d)", a->aux, a->block_len);
+    if (a->pattern == T5A_PATTERN_TGLOBAL && (a->aux <= 0 || a->n_side < 0))
+        return fail(T5A_ERR_PATTERN, "transient-global needs aux > 0 and n_side >= 0 (aux=%d n_side=%d)", a->aux, a->n_side);
+    if (a->B == 0 || a->L == 0) return T5A_OK;
+    if ((rc = check_tensor("q", a->q, a->q_strides, 3, unit))) return rc;
+    if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
+    if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
+    if ((rc = check_tensor("o", a->o, a->o_strides, 3, unit))) return rc;
+    if (a->pattern == T5A_PATTERN_TGLOBAL && a->n_side > 0) {
+        if ((rc = check_tensor("side_k", a->side_k, a->side_k_strides, 3, unit))) return rc;
+        if ((rc = check_tensor("side_v", a->side_v, a->side_v_strides, 3, unit))) return rc;
+    }
+    FwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
+    p.side_k = a->side_k; p.side_v = a->side_v;
+    p.q_sb = a->q_strides[0]; p.q_sh = a->q_strides[1]; p.q_sr = a->q_strides[2];
+    p.k_sb = a->k_strides[0]; p.k_sh = a->k_strides[1]; p.k_sr = a->k_strides[2];
+    p.v_sb = a->v_strides[0]; p.v_sh = a->v_strides[1]; p.v_sr = a->v_strides[2];
+    p.o_sb = a->o_strides[0]; p.o_sh = a->o_strides[1]; p.o_sr = a->o_strides[2];
+    p.sk_sb = a->side_k_strides[0]; p.sk_sh = a->side_k_strides[1]; p.sk_sr = a->side_k_strides[2];
+    p.sv_sb = a->side_v_strides[0]; p.sv_sh = a->side_v_strides[1]; p.sv_sr = a->side_v_strides[2];
+    p.B = a->B; p.H = a->H; p.M = a->L; p.N = a->L;
+    p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
+    p.c1 = a->sm_scale * kLog2e;
+    if ((rc = fill_bias(a->bias, true, &p))) return rc;
+    hipStream_t s = (hipStream_t)stream;
+
+    if (a->pattern == T5A_PATTERN_BLOCK) {
+        if (a->L < a->block_len) {
+            // shorter than one block: the reference degenerates to full attention (attentions.py:752, :691)
+            p.tiles_per_seq = (a->L + 127) / 128;
+            p.total_items = p.tiles_per_seq * a->H * a->B;
+            return finish(launch_fwd(p, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, short)");
+        }
+        // pass 1: rows >= G attend [global tokens | own block]
+        const int nblk = (a->L + a->block_len - 1) / a->block_len;
+        p.tiles_per_seq = nblk * ((a->block_len + 127) / 128);
+        p.total_items = p.tiles_per_seq * a->H * a->B;
+        rc = finish(launch_fwd(p, a->dtype, a->D, kBlock, false, s), "t5a_fwd_sparse(block)");
+        if (rc || a->aux == 0) return rc;
+        // pass 2: the G global queries attend every key; positions are absolute, so M is
+        // clipped to G rows of the same tensors (rel = j - i, no end alignment)
+        FwdParams g = p;
+        g.M = a->aux < a->L ? a->aux : a->L;
+        g.N = a->L;
+        g.tiles_per_seq = (g.M + 127) / 128;
+        g.total_items = g.tiles_per_seq * a->H * a->B;
+        g.align_end = 0;
+        return finish(launch_fwd(g, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, global rows)");
+    }
+    p.tiles_per_seq = (a->L + 127) / 128;
+    p.total_items = p.tiles_per_seq * a->H * a->B;
+    return finish(launch_fwd(p, a->dtype, a->D, a->pattern == T5A_PATTERN_LOCAL ? kLocal : kTGlobal, false, s), "t5a_fwd_sparse");
+}
+
+int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, int32_t num_splits) {
+    if (B < 0 || H < 0 || M < 0 || D < 0 || num_splits < 0) return -1;
+    return (int64_t)B * H * num_splits * M * ((int64_t)D + 2) * (int64_t)sizeof(float);
+}
+
+int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    if (a->B < 0 || a->H <= 0 || a->M < 0 || a->N < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d M=%d N=%d", a->B, a->H, a->M, a->N);
+    if (a->num_splits < 1 || a->num_splits > 65535) return fail(T5A_ERR_SHAPE, "num_splits=%d out of range", a->num_splits);
+    if (a->H > 65535 || (int64_t)a->B * ((a->M + 3) / 4 + 1) > 65535) return fail(T5A_ERR_SHAPE, "B*M or H too large for the launch grid");
+    if (a->B == 0 || a->M == 0) return T5A_OK;
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if ((rc = check_tensor("q", a->q, a->q_strides, 3, unit))) return rc;
+    if ((rc = check_tensor("o", a->o, a->o_strides, 3, 1))) return rc;
+    if (a->N > 0) {
+        if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
+        if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
+    }
+    const int64_t need = t5a_splitk_workspace_bytes(a->B, a->H, a->M, a->D, a->num_splits);
+    if (a->workspace == nullptr || a->workspace_bytes < need)
+        return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)a->workspace_bytes);
+    if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+    SplitKParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.bias = a->attn_bias;
+    const int64_t rows = (int64_t)a->B * a->H * a->num_splits * a->M;
+    p.part_o = reinterpret_cast<float*>(a->workspace);
+    p.part_l = p.part_o + rows * a->D;
+    p.part_m = p.part_l + rows;
+    p.q_sb = a->q_strides[0]; p.q_sh = a->q_strides[1]; p.q_sr = a->q_strides[2];
+    p.k_sb = a->k_strides[0]; p.k_sh = a->k_strides[1]; p.k_sr = a->k_strides[2];
+    p.v_sb = a->v_strides[0]; p.v_sh = a->v_strides[1]; p.v_sr = a->v_strides[2];
+    p.o_sb = a->o_strides[0]; p.o_sh = a->o_strides[1]; p.o_sr = a->o_strides[2];
+    p.b_sb = a->bias_strides[0]; p.b_sh = a->bias_strides[1]; p.b_sr = a->bias_strides[2]; p.b_sc = a->bias_strides[3];
+    p.B = a->B; p.H = a->H; p.M = a->M; p.N = a->N; p.S = a->num_splits;
+    p.sm_scale = a->sm_scale;
+    return finish(launch_splitk(p, a->dtype, a->D, (hipStream_t)stream), "t5a_fwd_splitk");
+}
+
+}  // extern "C"

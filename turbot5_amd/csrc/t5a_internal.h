@@ -1,0 +1,68 @@
+// Internal declarations shared by the host API and the HIP kernels of libt5attn.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/t5attn.h"
+
+namespace t5a {
+
+constexpr int kMaxThresholds = 128;   // supports num_buckets up to 256
+constexpr int kMaxSaturation = 1024;  // largest distance at which buckets still change
+
+// Integer description of the T5 bucket function, derived on the host from the
+// per-distance table so that device code never evaluates a logarithm.
+// For distance d >= max_exact the bucket is max_exact + #{t : thr[t] <= d}.
+struct BucketSpec {
+    int bidirectional;
+    int nb;         // buckets per direction (num_buckets/2 if bidirectional)
+    int max_exact;  // nb / 2
+    int n_thr;
+    int sat;        // every |rel| >= sat maps to the last bucket of its side
+    int thr[kMaxThresholds];
+};
+
+enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3 };
+
+struct FwdParams {
+    const void* q; const void* k; const void* v; void* o; float* lse;
+    const void* side_k; const void* side_v;
+    int64_t q_sb, q_sh, q_sr;
+    int64_t k_sb, k_sh, k_sr;
+    int64_t v_sb, v_sh, v_sr;
+    int64_t o_sb, o_sh, o_sr;
+    int64_t sk_sb, sk_sh, sk_sr;
+    int64_t sv_sb, sv_sh, sv_sr;
+    int64_t lse_sb, lse_sh, lse_sr;
+    const int32_t* cu_q; const int32_t* cu_k;   // non-null: packed variable-length batch
+    int B, H, M, N;
+    int tiles_per_seq;   // q tiles per (batch, head) when not packed
+    int total_items;     // number of (q tile, head, batch) work items (upper bound when packed)
+    float c1;            // sm_scale * log2(e)
+    const void* table; int table_dtype; int64_t t_sbucket, t_shead;
+    int block_len, aux, n_side;
+    int align_end;       // 1: query i sits at key position i + N - M (KV-cache alignment); 0: at i
+    BucketSpec bs;
+};
+
+// host side (api.cpp)
+int fail(int code, const char* fmt, ...);
+int make_bucket_spec(bool bidirectional, int num_buckets, int max_distance, BucketSpec* out);
+
+// launchers (attn_fwd.hip, splitk.hip)
+hipError_t launch_fwd_bf16(const FwdParams& p, int D, int mode, bool causal, hipStream_t stream);
+hipError_t launch_fwd_f16(const FwdParams& p, int D, int mode, bool causal, hipStream_t stream);
+hipError_t launch_fwd_f32(const FwdParams& p, int D, int mode, bool causal, hipStream_t stream);
+
+struct SplitKParams {
+    const void* q; const void* k; const void* v; void* o;
+    const float* bias;
+    float* part_o; float* part_l; float* part_m;
+    int64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr, v_sb, v_sh, v_sr, o_sb, o_sh, o_sr;
+    int64_t b_sb, b_sh, b_sr, b_sc;
+    int B, H, M, N, S;
+    float sm_scale;
+};
+hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t stream);
+
+}  // namespace t5a

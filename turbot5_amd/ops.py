@@ -1,0 +1,264 @@
+"""Function-level API of the attention hot path, with the reference's signatures.
+
+``flash_attention_with_fusing_bias`` and ``flash_attention_with_fusing_bias_varlen``
+keep the names, argument order and defaults of the reference
+(src/turbot5/ops/fused_bias_attention.py:876-890, varlen_fused_bias_attn.py:870-889);
+``flash_attn_v2_fwd`` keeps those of src/turbot5/ops/flash_decoding.py:6.
+All of them launch hand-written HIP kernels through libt5attn.so; tensors must
+live on a ROCm device.  Forward only: the outputs carry no autograd graph.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+
+_DTYPES = {torch.bfloat16: L.T5A_BF16, torch.float32: L.T5A_F32, torch.float16: L.T5A_F16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected bfloat16, float16 or float32") from None
+
+
+def _check_inputs(q, k, v):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("q, k, v must be on a ROCm device: this path has no CPU implementation")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError(f"q, k, v dtypes differ: {q.dtype}, {k.dtype}, {v.dtype}")
+    Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Dq == Dk == Dv                       # fused_bias_attention.py:827
+    assert Dk in {16, 32, 64, 128}              # fused_bias_attention.py:828
+
+
+def _unit(t: torch.Tensor) -> int:
+    return 4 if t.dtype == torch.float32 else 8
+
+
+def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
+    """The kernels need head_dim contiguous, 16-byte aligned rows; copy only when that fails."""
+    u = _unit(t)
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % u == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
+def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_distance: int, ref: torch.Tensor):
+    b = L.T5ABias()
+    if bias is None:
+        b.table = None
+        return b, None
+    if bias.dim() != 2 or bias.shape[0] != num_buckets or bias.shape[1] != H:
+        raise ValueError(f"bias table must be (NUM_BUCKETS={num_buckets}, H={H}), got {tuple(bias.shape)}")
+    if bias.device != ref.device:
+        raise RuntimeError("bias table must be on the same device as q")
+    table = bias.detach()
+    if table.dtype not in _DTYPES:
+        table = table.float()
+    b.table = table.data_ptr()
+    b.table_dtype = _DTYPES[table.dtype]
+    b.num_buckets = num_buckets
+    b.max_distance = max_distance
+    b.stride_bucket = table.stride(0)
+    b.stride_head = table.stride(1)
+    return b, table   # keep `table` alive until the launch has been queued
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _strides3(t):
+    return (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
+                                     return_lse: bool = False):
+    """FlashAttention forward with the T5 relative-position bias computed inside the kernel.
+
+    q (B,H,M,D); k, v (B,H,N,D), any batch/head/row strides; ``bias`` is the
+    (NUM_BUCKETS, H) table or None.  ``causal`` selects the causal mask and the
+    unidirectional buckets together.  ``sm_scale=None`` means 1/sqrt(D).  Returns
+    a tensor shaped and strided like q (``empty_like``), plus the (B,H,M) fp32
+    log-sum-exp when ``return_lse``.
+    """
+    _check_inputs(q, k, v)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    if k.shape[0] != B or k.shape[1] != H or v.shape != k.shape:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    o = torch.empty_like(q_)
+    lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32) if return_lse else None
+    a = L.T5ADenseArgs()
+    a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
+    a.lse = lse.data_ptr() if lse is not None else None
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q_), _strides3(k_), _strides3(v_), _strides3(o)
+    a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
+    a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    with torch.cuda.device(q.device):
+        L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
+    return (o, lse) if return_lse else o
+
+
+def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                            causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
+                                            return_lse: bool = False):
+    """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
+
+    Positions restart at 0 in every sequence.  No host synchronisation: the
+    work list is derived on the device from ``cu_seqlens``.
+    """
+    _check_inputs(q, k, v)
+    total_q, H, D = q.shape
+    total_k = k.shape[0]
+    if k.shape[1] != H or v.shape != k.shape:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    B = cu_seqlens_q.numel() - 1
+    if cu_seqlens_k.numel() != B + 1:
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must have the same length")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    cq = cu_seqlens_q.to(device=q.device, dtype=torch.int32).contiguous()
+    ck = cq if cu_seqlens_k is cu_seqlens_q else cu_seqlens_k.to(device=q.device, dtype=torch.int32).contiguous()
+    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    o = torch.empty_like(q_)
+    lse = torch.empty((total_q, H), device=q.device, dtype=torch.float32) if return_lse else None
+    a = L.T5AVarlenArgs()
+    a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
+    a.lse = lse.data_ptr() if lse is not None else None
+    for name, t in (("q_strides", q_), ("k_strides", k_), ("v_strides", v_), ("o_strides", o)):
+        setattr(a, name, (C.c_int64 * 2)(t.stride(0), t.stride(1)))
+    a.cu_seqlens_q, a.cu_seqlens_k = cq.data_ptr(), ck.data_ptr()
+    a.dtype, a.B, a.H, a.D = _dtype_code(q), B, H, D
+    a.total_q, a.total_k = total_q, total_k
+    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    with torch.cuda.device(q.device):
+        L.check(L.load().t5a_fwd_varlen(C.byref(a), _stream(q)))
+    return (o, lse) if return_lse else o
+
+
+def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
+            NUM_BUCKETS=32, MAX_DISTANCE=128):
+    _check_inputs(q, k, v)
+    B, H, Lq, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("sparse self-attention needs q, k, v of one shape")
+    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    o = torch.empty_like(q_)
+    a = L.T5ASparseArgs()
+    a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q_), _strides3(k_), _strides3(v_), _strides3(o)
+    keep_side = None
+    if pattern == L.PATTERN_TGLOBAL:
+        if side_k is None or side_v is None or side_k.shape != side_v.shape:
+            raise ValueError("transient-global attention needs side_k and side_v of one shape")
+        if side_k.shape[0] != B or side_k.shape[1] != H or side_k.shape[3] != D or side_k.dtype != q.dtype:
+            raise ValueError(f"side_k must be (B,H,n_side,D) in {q.dtype}, got {tuple(side_k.shape)} {side_k.dtype}")
+        sk, sv = _kernel_ready(side_k.detach()), _kernel_ready(side_v.detach())
+        keep_side = (sk, sv)
+        a.side_k, a.side_v = sk.data_ptr(), sv.data_ptr()
+        a.side_k_strides, a.side_v_strides = _strides3(sk), _strides3(sv)
+        a.n_side = sk.shape[2]
+    a.dtype, a.B, a.H, a.L, a.D = _dtype_code(q), B, H, Lq, D
+    a.pattern, a.block_len, a.aux = pattern, int(block_len), int(aux)
+    a.sm_scale = float(sm_scale)
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    with torch.cuda.device(q.device):
+        L.check(L.load().t5a_fwd_sparse(C.byref(a), _stream(q)))
+    return o
+
+
+def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128):
+    """Sliding-window self-attention: key j visible to query i iff |j-i| < block_len, bias bucket(j-i).
+
+    The op of T5LocalAttention (src/turbot5/model/attentions.py:583-638) without
+    blocking, K/V triplication or a bias tensor.  q,k,v (B,H,L,D)."""
+    return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE)
+
+
+def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
+                                     MAX_DISTANCE=128):
+    """Block attention with ``n_global`` leading global tokens, the op of T5BlockAttention
+    (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout."""
+    return _sparse(L.PATTERN_BLOCK, q, k, v, bias, block_len, n_global, None, None, sm_scale, NUM_BUCKETS,
+                   MAX_DISTANCE)
+
+
+def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
+                                                sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128):
+    """Sliding window plus side tokens, the op of T5TransientGlobalAttention
+    (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D)."""
+    return _sparse(L.PATTERN_TGLOBAL, q, k, v, bias, block_len, global_block_size, side_k, side_v, sm_scale,
+                   NUM_BUCKETS, MAX_DISTANCE)
+
+
+def default_num_splits(B: int, H: int, N: int, device=None) -> int:
+    """Enough splits to give every compute unit a few workgroups, at least 256 keys per split."""
+    cus = 256
+    if device is not None and torch.cuda.is_available():
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+    want = max(1, (4 * cus + B * H - 1) // max(1, B * H))
+    return int(max(1, min(want, max(1, N // 256), 64)))
+
+
+def flash_attn_v2_fwd(q, k, v, bias, causal, sm_scale, NUM_SPLITS=None, BLOCK_M=None, BLOCK_N=None, num_warps=None,
+                      num_stages=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Flash-decoding split-K forward (src/turbot5/ops/flash_decoding.py:6-55).
+
+    q (B,H,M,D) with small M; k, v (B,H,N,D); ``bias`` an additive tensor
+    broadcastable to (B,H,M,N) or None; ``causal`` is accepted and unused, as in
+    the reference; the tile arguments are accepted and ignored (fixed in the
+    kernel).  Returns (res, L, ml): res (B,H,M,D) fp32 merged output, L and ml
+    the per-split sums of exp and maxima, (B,H,S) when M == 1 else (B,H,S,M).
+    """
+    out, part_l, part_m = _splitk(q, k, v, bias, sm_scale, NUM_SPLITS, out_dtype=torch.float32)
+    if q.shape[2] == 1:
+        part_l, part_m = part_l.squeeze(-1), part_m.squeeze(-1)
+    return out, part_l, part_m
+
+
+def flash_decoding_attention(q, k, v, bias=None, sm_scale=1.0, num_splits=None) -> torch.Tensor:
+    """Split-K attention returning only the merged output in q's dtype."""
+    return _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype=q.dtype)[0]
+
+
+def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype):
+    _check_inputs(q, k, v)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    S = int(num_splits) if num_splits else default_num_splits(B, H, N, q.device)
+    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    lib = L.load()
+    nbytes = lib.t5a_splitk_workspace_bytes(B, H, M, D, S)
+    ws = torch.empty(max(nbytes, 16) // 4, device=q.device, dtype=torch.float32)
+    o = torch.empty((B, H, M, D), device=q.device, dtype=q.dtype)
+    a = L.T5ASplitKArgs()
+    a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q_), _strides3(k_), _strides3(v_), _strides3(o)
+    keep = None
+    if bias is not None:
+        keep = bias.detach().float().expand(B, H, M, N)
+        a.attn_bias = keep.data_ptr()
+        a.bias_strides = (C.c_int64 * 4)(*keep.stride())
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
+    a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
+    a.num_splits, a.sm_scale = S, float(sm_scale)
+    with torch.cuda.device(q.device):
+        L.check(lib.t5a_fwd_splitk(C.byref(a), _stream(q)))
+    rows = B * H * S * M
+    part_l = ws[rows * D: rows * D + rows].view(B, H, S, M)
+    part_m = ws[rows * D + rows: rows * D + 2 * rows].view(B, H, S, M)
+    return (o if out_dtype == q.dtype else o.to(out_dtype)), part_l, part_m
