@@ -5,11 +5,18 @@
 // owns 128 query rows (32 per wavefront) of one (batch, head) and walks over
 // at most two key segments in tiles of 64 keys.  Per tile:
 //
-//   S^T = K Q^T      32x32 MFMA with K rows as the A operand, so that every
+//   S^T = K Q^T + C  32x32 MFMA with K rows as the A operand, so that every
 //                    lane owns ONE query column and 16 keys per 32x32 block:
 //                    the softmax row reductions stay inside the lane, with one
-//                    cross-half exchange per tile.
-//   P   = exp2(..)   online softmax in base 2, running max / sum per lane.
+//                    cross-half exchange per tile.  Q is pre-multiplied by
+//                    sm_scale*log2(e); the accumulator input C carries
+//                    (bias - running max), so the MFMA result is directly the
+//                    exp2 argument.
+//   P   = exp2(S^T)  online softmax in base 2.  The running max is only raised
+//                    when a tile exceeds it by more than 2^8 (the sums and the
+//                    output are normalised by the same stale max, so the
+//                    result is unchanged), which keeps the rescale off the
+//                    common path.
 //   O^T += V^T P^T   the S^T accumulators are already laid out as the B
 //                    operand (for 16-bit types after a key permutation that is
 //                    baked into the LDS layout of V^T), so P stays in registers.
@@ -18,15 +25,18 @@
 // LDS, V tiles transposed (head_dim x keys), both with an XOR swizzle on
 // 16-byte chunks.  fp32 inputs use v_mfma_f32_32x32x2_f32 (one float per lane
 // and operand) with K and V row-major and P kept in fp32.  Tiles are double
-// buffered and filled from registers that were loaded from HBM during the
-// previous tile's math.
+// buffered and filled from registers that were loaded from HBM (buffer loads,
+// rows past the end of a segment read as zero) during the previous tile's math.
 //
 // The T5 relative-position bias is not materialised.  Each workgroup expands
 // its head's column of the (num_buckets, H) table into a distance-indexed LUT
-// in LDS covering [-sat, sat] (sat = distance at which the buckets saturate).
-// Key tiles whose distances are all beyond saturation take the FAST path where
-// the bias is one scalar folded into the exp2 argument; only tiles near the
-// diagonal (or needing a mask) take the GENERAL path with per-element lookups.
+// in LDS covering the distances at which buckets still change; for causal
+// attention the LUT holds -inf for every future key, so the diagonal needs no
+// separate mask.  Four copies of the LUT, shifted by 0..3 entries, let a lane
+// fetch the biases of four consecutive keys with one aligned 16-byte read,
+// straight into the MFMA accumulator input.  Key tiles whose distances are all
+// beyond saturation use a per-lane constant instead.  Per-element masking is
+// left to the few tiles that straddle the end of a segment or a window edge.
 //
 // Sparsity patterns are tile skipping: the key segments of a work item are
 // computed from integer positions; nothing outside them is loaded.
@@ -39,8 +49,12 @@ typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 template <typename T> struct Elem;
 template <> struct Elem<__bf16> {
@@ -48,11 +62,30 @@ template <> struct Elem<__bf16> {
     static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // sum of the eight values as the matrix core will see them (rounded to bf16)
+    static __device__ __forceinline__ float sum8(v8 x, float acc) {
+        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bf16x2 pr = {x[2 * i], x[2 * i + 1]};
+            acc = __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false);
+        }
+        return acc;
+    }
 };
 template <> struct Elem<_Float16> {
     using v8 = f16x8; using v4 = f16x4;
     static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float sum8(v8 x, float acc) {
+        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f16x2 pr = {x[2 * i], x[2 * i + 1]};
+            acc = __builtin_amdgcn_fdot2(pr, one, acc, false);
+        }
+        return acc;
     }
 };
 template <> struct Elem<float> {
@@ -66,7 +99,8 @@ constexpr int BM = 128;      // query rows per workgroup
 constexpr int BN = 64;       // keys per tile
 constexpr int NTHREADS = 256;
 constexpr int NT = BN / 32;  // 32-key blocks per tile
-constexpr float kNegBig = -1.0e30f;
+constexpr int LUT_PAD = 8;   // saturated entries kept on the left of the distance LUT
+constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 
 __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
     int out = 0, d;
@@ -84,8 +118,23 @@ __device__ __forceinline__ float load_table(const void* table, int dtype, int64_
     return static_cast<float>(reinterpret_cast<const _Float16*>(table)[off]);
 }
 
-__device__ __forceinline__ float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
-__device__ __forceinline__ float xhalf_sum(float x) { return x + __shfl_xor(x, 32); }
+// max / sum over the two lanes (l, l^32) that share a query row; the swap
+// exchanges the upper half of one operand with the lower half of the other, so
+// combining both results is symmetric in the halves.
+__device__ __forceinline__ float xhalf_max(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xhalf_sum(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
 
 template <typename T, int D>
 struct Geometry {
@@ -107,8 +156,14 @@ struct Geometry {
     static constexpr size_t kTileBytes = (size_t)(2 * K_TILE + 2 * V_TILE) * sizeof(T);
 };
 
+// floats per shifted copy of the distance LUT (host and device agree through this)
+__host__ __device__ inline int lut_quads(int sat, bool causal) {
+    const int e_right = sat + LUT_PAD + (causal ? 1 : sat);   // first index of the right-saturated part
+    return (e_right + 3) / 4 + 2;                              // quads 0 .. ymax, ymax = quads - 1
+}
+
 template <typename T, int D, int MODE, bool CAUSAL>
-__global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
     using v8 = typename E::v8;
@@ -117,15 +172,16 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
     constexpr int EPC = G::EPC, KS = G::KS, DT = G::DT, VROWS = G::VROWS, CH = G::CH, SW = G::SW;
     constexpr int K_CHUNKS = G::K_CHUNKS, K_PER_T = G::K_PER_T, V_UNITS = G::V_UNITS, V_PER_T = G::V_PER_T;
     constexpr int KSTR = G::KSTR, K_TILE = G::K_TILE, V_TILE = G::V_TILE;
+    constexpr int ES = sizeof(T);
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     T* Vs = reinterpret_cast<T*>(smem);         // [2][V_TILE]
     T* Ks = Vs + 2 * V_TILE;                    // [2][K_TILE]
-    float* lut = reinterpret_cast<float*>(Ks + 2 * K_TILE);
+    float* lut = reinterpret_cast<float*>(Ks + 2 * K_TILE);   // [4][4*quads]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 31;
     const int hh = lane >> 5;
 
@@ -199,13 +255,13 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
     // position is its index j; the query position depends on the kind:
     //   0: i + P     1: i % block_len + G (block pattern, global keys)     2: i / aux (side tokens)
     const T* seg_k[2]; const T* seg_v[2];
-    int64_t seg_ksr[2], seg_vsr[2];
+    int seg_ksr[2], seg_vsr[2];      // row strides in bytes
     int seg_start[2], seg_end[2], seg_lend[2], seg_kind[2], seg_win[2];
     int nseg = 1;
     seg_k[0] = reinterpret_cast<const T*>(p.k) + k_off;
     seg_v[0] = reinterpret_cast<const T*>(p.v) + v_off;
-    seg_ksr[0] = p.k_sr; seg_vsr[0] = p.v_sr;
-    seg_k[1] = seg_k[0]; seg_v[1] = seg_v[0]; seg_ksr[1] = p.k_sr; seg_vsr[1] = p.v_sr;
+    seg_ksr[0] = (int)p.k_sr * ES; seg_vsr[0] = (int)p.v_sr * ES;
+    seg_k[1] = seg_k[0]; seg_v[1] = seg_v[0]; seg_ksr[1] = seg_ksr[0]; seg_vsr[1] = seg_vsr[0];
     seg_start[0] = 0; seg_end[0] = 0;
     seg_start[1] = seg_end[1] = seg_lend[1] = 0; seg_kind[1] = 0; seg_win[1] = 0;
     seg_kind[0] = 0; seg_win[0] = 0; seg_lend[0] = Nseq;
@@ -219,7 +275,7 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
             nseg = 2;
             seg_k[1] = reinterpret_cast<const T*>(p.side_k) + (int64_t)b * p.sk_sb + (int64_t)h * p.sk_sh;
             seg_v[1] = reinterpret_cast<const T*>(p.side_v) + (int64_t)b * p.sv_sb + (int64_t)h * p.sv_sh;
-            seg_ksr[1] = p.sk_sr; seg_vsr[1] = p.sv_sr;
+            seg_ksr[1] = (int)p.sk_sr * ES; seg_vsr[1] = (int)p.sv_sr * ES;
             seg_end[1] = p.n_side; seg_lend[1] = p.n_side; seg_kind[1] = 2;
         }
     } else {  // kBlock
@@ -233,25 +289,42 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
     seg_nt[0] = max(0, seg_end[0] - seg_start[0] + BN - 1) / BN;
     seg_nt[1] = nseg > 1 ? max(0, seg_end[1] - seg_start[1] + BN - 1) / BN : 0;
     const int ntiles = seg_nt[0] + seg_nt[1];
+    __amdgpu_buffer_rsrc_t seg_krs[2], seg_vrs[2];
+#pragma unroll
+    for (int sg = 0; sg < 2; ++sg) {
+        const int rows = min(seg_lend[sg], seg_end[sg]);   // rows at or past this read as zero
+        seg_krs[sg] = make_rsrc(seg_k[sg], rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_ksr[sg] + D * ES : 0u);
+        seg_vrs[sg] = make_rsrc(seg_v[sg], rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_vsr[sg] + D * ES : 0u);
+    }
 
     // ---------------------------------------------------------------- bias LUT
     const bool has_bias = p.table != nullptr;
-    const int sat = p.bs.sat;
-    if (has_bias) {
-        const float log2e = 1.4426950408889634f;
-        for (int idx = tid; idx <= 2 * sat; idx += NTHREADS) {
-            const int bk = bucket_of(p.bs, idx - sat);
-            lut[idx] = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+    const bool has_lut = has_bias || CAUSAL;
+    const int sat = has_bias ? p.bs.sat : 0;
+    const int padl = sat + LUT_PAD;                       // LUT index of rel = 0
+    const int quads = lut_quads(sat, CAUSAL);
+    const int qlen = 4 * quads;
+    const float log2e = 1.4426950408889634f;
+    if (has_lut) {
+        for (int idx = tid; idx < 4 * qlen; idx += NTHREADS) {
+            const int a = idx / qlen, i = idx - a * qlen;
+            const int rel = i + a - padl;
+            float val = 0.f;
+            if (has_bias)
+                val = load_table(p.table, p.table_dtype,
+                                 (int64_t)bucket_of(p.bs, rel) * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+            if (CAUSAL && rel > 0) val = -INFINITY;
+            lut[idx] = val;
         }
     }
     if (D < 32) {  // the part of V past head_dim feeds the MFMA: keep it zero
         for (int idx = tid; idx < 2 * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
     }
     __syncthreads();
-    const float c_neg = has_bias ? lut[0] : 0.f;
-    const float c_pos = has_bias ? lut[2 * sat] : 0.f;
+    const float c_neg = has_bias ? lut[0] : 0.f;                 // every key far before the query
+    const float c_pos = has_bias ? lut[qlen - 1] : 0.f;          // every key far after it (non-causal)
 
-    // ---------------------------------------------------------------- Q fragments
+    // ---------------------------------------------------------------- Q fragments (pre-scaled)
     const int iw0 = i0 + wave * 32;      // first row of this wavefront
     const int iw1 = iw0 + 31;
     const int irow = iw0 + lr;           // this lane's query row
@@ -262,20 +335,24 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
         for (int c = 0; c < D / 4; ++c) {
             f32x4 x = {0.f, 0.f, 0.f, 0.f};
             if (row_ok) x = *reinterpret_cast<const f32x4*>(qp + (int64_t)irow * p.q_sr + 4 * c);
-            qf[2 * c] = hh ? x[1] : x[0];
-            qf[2 * c + 1] = hh ? x[3] : x[2];
+            qf[2 * c] = (hh ? x[1] : x[0]) * p.c1;
+            qf[2 * c + 1] = (hh ? x[3] : x[2]) * p.c1;
         }
     } else {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            if (row_ok) qf[s] = *reinterpret_cast<const v8*>(qp + (int64_t)irow * p.q_sr + 16 * s + 8 * hh);
-            else { for (int x = 0; x < 8; ++x) qf[s][x] = (T)0.0f; }
+            v8 x;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (T)0.0f;
+            if (row_ok) x = *reinterpret_cast<const v8*>(qp + (int64_t)irow * p.q_sr + 16 * s + 8 * hh);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)x[e] * p.c1);
         }
     }
 
     // ---------------------------------------------------------------- tile staging
-    uint4 kreg[K_PER_T];
-    uint4 vreg[F32 ? V_PER_T : 2 * V_PER_T];   // 16-bit: four 8-byte rows per unit
+    u32x4 kreg[K_PER_T];
+    u32x4 vreg[F32 ? V_PER_T : 2 * V_PER_T];   // 16-bit: four 8-byte rows per unit
 
     auto tile_of = [&](int t, int& sg, int& j0) {
         sg = t >= seg_nt[0] ? 1 : 0;
@@ -283,40 +360,38 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
     };
     auto load_tile = [&](int t) {
         int sg, j0; tile_of(t, sg, j0);
-        const T* kp = seg_k[sg]; const T* vp = seg_v[sg];
-        const int64_t ksr = seg_ksr[sg], vsr = seg_vsr[sg];
-        const int lend = min(seg_lend[sg], seg_end[sg]);
+        const __amdgpu_buffer_rsrc_t krs = sg ? seg_krs[1] : seg_krs[0];
+        const __amdgpu_buffer_rsrc_t vrs = sg ? seg_vrs[1] : seg_vrs[0];
+        const int ksr = seg_ksr[sg], vsr = seg_vsr[sg];
+        // the whole byte offset goes into the vector operand: only that one is range checked
 #pragma unroll
         for (int c = 0; c < K_PER_T; ++c) {
             const int idx = tid + c * NTHREADS;
             const int row = idx / CH, ch = idx % CH;
-            const int j = j0 + row;
-            kreg[c] = make_uint4(0, 0, 0, 0);
-            if (idx < K_CHUNKS && j < lend) kreg[c] = *reinterpret_cast<const uint4*>(kp + (int64_t)j * ksr + ch * EPC);
+            if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS)
+                kreg[c] = __builtin_amdgcn_raw_buffer_load_b128(krs, (j0 + row) * ksr + ch * 16, 0, 0);
         }
         if constexpr (F32) {
 #pragma unroll
             for (int c = 0; c < V_PER_T; ++c) {
                 const int idx = tid + c * NTHREADS;
                 const int row = idx / CH, ch = idx % CH;
-                const int j = j0 + row;
-                vreg[c] = make_uint4(0, 0, 0, 0);
-                if (idx < V_UNITS && j < lend) vreg[c] = *reinterpret_cast<const uint4*>(vp + (int64_t)j * vsr + ch * EPC);
+                if (V_UNITS % NTHREADS == 0 || idx < V_UNITS)
+                    vreg[c] = __builtin_amdgcn_raw_buffer_load_b128(vrs, (j0 + row) * vsr + ch * 16, 0, 0);
             }
         } else {
 #pragma unroll
             for (int u = 0; u < V_PER_T; ++u) {
                 const int idx = tid + u * NTHREADS;
                 const int dg = idx % (D / 4), kg = idx / (D / 4);
-                uint2 r[4];
+                if (V_UNITS % NTHREADS == 0 || idx < V_UNITS) {
+                    u32x2 r[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = j0 + 4 * kg + i;
-                    r[i] = make_uint2(0, 0);
-                    if (idx < V_UNITS && j < lend) r[i] = *reinterpret_cast<const uint2*>(vp + (int64_t)j * vsr + 4 * dg);
+                    for (int i = 0; i < 4; ++i)
+                        r[i] = __builtin_amdgcn_raw_buffer_load_b64(vrs, (j0 + 4 * kg + i) * vsr + dg * 8, 0, 0);
+                    vreg[2 * u] = u32x4{r[0][0], r[0][1], r[1][0], r[1][1]};
+                    vreg[2 * u + 1] = u32x4{r[2][0], r[2][1], r[3][0], r[3][1]};
                 }
-                vreg[2 * u] = make_uint4(r[0].x, r[0].y, r[1].x, r[1].y);
-                vreg[2 * u + 1] = make_uint4(r[2].x, r[2].y, r[3].x, r[3].y);
             }
         }
     };
@@ -328,44 +403,45 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
             for (int c = 0; c < K_PER_T; ++c) {
                 const int idx = tid + c * NTHREADS;
                 const int row = idx / CH, ch = idx % CH;
-                if (idx < K_CHUNKS) {
+                if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS) {
                     float* dst = reinterpret_cast<float*>(ks) + row * KSTR + ch * 4;
-                    dst[0] = __uint_as_float(kreg[c].x); dst[1] = __uint_as_float(kreg[c].y);
-                    dst[2] = __uint_as_float(kreg[c].z); dst[3] = __uint_as_float(kreg[c].w);
+                    dst[0] = __uint_as_float(kreg[c][0]); dst[1] = __uint_as_float(kreg[c][1]);
+                    dst[2] = __uint_as_float(kreg[c][2]); dst[3] = __uint_as_float(kreg[c][3]);
                 }
             }
 #pragma unroll
             for (int c = 0; c < V_PER_T; ++c) {
                 const int idx = tid + c * NTHREADS;
                 const int row = idx / CH, ch = idx % CH;
-                if (idx < V_UNITS) *reinterpret_cast<uint4*>(vs + row * VROWS + ch * 4) = vreg[c];
+                if (V_UNITS % NTHREADS == 0 || idx < V_UNITS)
+                    *reinterpret_cast<u32x4*>(vs + row * VROWS + ch * 4) = vreg[c];
             }
         } else {
 #pragma unroll
             for (int c = 0; c < K_PER_T; ++c) {
                 const int idx = tid + c * NTHREADS;
                 const int row = idx / CH, ch = idx % CH;
-                if (idx < K_CHUNKS)
-                    *reinterpret_cast<uint4*>(ks + row * D + ((ch ^ (row & (SW - 1))) * 8)) = kreg[c];
+                if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS)
+                    *reinterpret_cast<u32x4*>(ks + row * D + ((ch ^ (row & (SW - 1))) * 8)) = kreg[c];
             }
 #pragma unroll
             for (int u = 0; u < V_PER_T; ++u) {
                 const int idx = tid + u * NTHREADS;
                 const int dg = idx % (D / 4), kg = idx / (D / 4);
-                if (idx < V_UNITS) {
+                if (V_UNITS % NTHREADS == 0 || idx < V_UNITS) {
                     // 4 keys x 4 dims -> 4 dims x 4 keys.  Key slots 4..7 and 8..11 of every 16 are
                     // swapped so that a lane's eight P values line up with one 16-byte V^T read.
                     const int pk = (kg & ~3) | ((kg & 1) << 1) | ((kg >> 1) & 1);
-                    const uint4 a = vreg[2 * u], c2 = vreg[2 * u + 1];   // keys (0,1) and (2,3): {x,y | z,w}
-                    uint2 y[4];
-                    y[0] = make_uint2((a.x & 0xffffu) | (a.z << 16), (c2.x & 0xffffu) | (c2.z << 16));
-                    y[1] = make_uint2((a.x >> 16) | (a.z & 0xffff0000u), (c2.x >> 16) | (c2.z & 0xffff0000u));
-                    y[2] = make_uint2((a.y & 0xffffu) | (a.w << 16), (c2.y & 0xffffu) | (c2.w << 16));
-                    y[3] = make_uint2((a.y >> 16) | (a.w & 0xffff0000u), (c2.y >> 16) | (c2.w & 0xffff0000u));
+                    const u32x4 a = vreg[2 * u], c2 = vreg[2 * u + 1];   // keys (0,1) and (2,3)
+                    u32x2 y[4];
+                    y[0] = u32x2{(a[0] & 0xffffu) | (a[2] << 16), (c2[0] & 0xffffu) | (c2[2] << 16)};
+                    y[1] = u32x2{(a[0] >> 16) | (a[2] & 0xffff0000u), (c2[0] >> 16) | (c2[2] & 0xffff0000u)};
+                    y[2] = u32x2{(a[1] & 0xffffu) | (a[3] << 16), (c2[1] & 0xffffu) | (c2[3] << 16)};
+                    y[3] = u32x2{(a[1] >> 16) | (a[3] & 0xffff0000u), (c2[1] >> 16) | (c2[3] & 0xffff0000u)};
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         const int d = 4 * dg + c;
-                        *reinterpret_cast<uint2*>(vs + d * BN + (((pk >> 1) ^ (d & 7)) * 8) + (pk & 1) * 4) = y[c];
+                        *reinterpret_cast<u32x2*>(vs + d * BN + (((pk >> 1) ^ (d & 7)) * 8) + (pk & 1) * 4) = y[c];
                     }
                 }
             }
@@ -378,8 +454,13 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
-    float m_run = kNegBig;   // running max (base-2 units); finite, so exp2(m_run - m_new) is never NaN
+    float m_run = 0.f;       // running max (base-2 units), meaningful once `started`
     float l_run = 0.f;       // running sum over this lane's half of the keys
+    bool started = false;    // a finite score has been seen for this row
+    f32x16 cm;               // accumulator input of tiles with a constant bias: cb - m_run in every slot
+    float cb_cur = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cm[r] = 0.f;
 
     if (ntiles > 0) { load_tile(0); store_tile(0); }
     __syncthreads();
@@ -404,23 +485,42 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
         if (win) skip = skip || (rel_max <= -p.block_len) || (rel_min >= p.block_len);
 
         if (!skip) {
-            bool general = (j0 + BN > s_end) || !(p.c1 > 0.f);
-            if (CAUSAL) general = general || (rel_max > 0);
-            if (win) general = general || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
-            float cb = 0.f;
-            if (has_bias) {
-                if (rel_max <= -sat) cb = c_neg;
-                else if (rel_min >= sat) cb = c_pos;
-                else general = true;
+            const bool left_sat = rel_max <= -sat && (!CAUSAL || rel_max <= 0);
+            const bool right_sat = !CAUSAL && rel_min >= sat;
+            const bool use_lut = has_lut && !(left_sat || right_sat);
+            bool need_mask = j0 + BN > s_end;
+            if (win) need_mask = need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
+
+            // ---- accumulator input: bias - running max
+            f32x16 st[NT];
+            if (use_lut) {
+                const int e0 = j0 + 4 * hh - qpos + padl;
+                const float* lb = lut + (e0 & 3) * qlen;
+                const int y0 = e0 >> 2;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
+                        const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
+                    }
+            } else {
+                const float cb = has_bias ? (left_sat ? c_neg : c_pos) : 0.f;
+                if (cb != cb_cur) {   // wavefront-uniform: the tile moved to the other side of the diagonal
+                    cb_cur = cb;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) cm[r] = cb - m_run;
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) st[nt] = cm;
             }
 
-            // ---- S^T = K Q^T
+            // ---- S^T = K Q^T + C
             const T* ks = Ks + buf * K_TILE;
-            f32x16 st[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) st[nt][r] = 0.f;
                 const int row = 32 * nt + lr;
 #pragma unroll
                 for (int s = 0; s < KS; ++s) {
@@ -433,78 +533,59 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
                 }
             }
 
-            // ---- online softmax (base 2)
-            float m_new;
-            float rsum = 0.f;
-            if (!general) {
-                float mx = st[0][0];
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[nt][r]);
-                mx = xhalf_max(mx);
-                m_new = fmaxf(m_run, fmaf(mx, p.c1, cb));
-                const float off = cb - m_new;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float e = __builtin_amdgcn_exp2f(fmaf(st[nt][r], p.c1, off));
-                        st[nt][r] = e;
-                        rsum += e;
-                    }
-            } else {
-                float mx = -INFINITY;
+            if (need_mask) {   // keys past the end of the segment, or outside the window
                 const int jl = j0 + 4 * hh;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int j = jl + 32 * nt + 8 * (r >> 2) + (r & 3);
-                        const int rel = j - qpos;
-                        float bias = 0.f;
-                        if (has_bias) bias = lut[min(max(rel, -sat), sat) + sat];
-                        float tt = fmaf(st[nt][r], p.c1, bias);
                         bool ok = j < s_end;
-                        if (CAUSAL) ok = ok && rel <= 0;
-                        if (win) ok = ok && rel < p.block_len && rel > -p.block_len;
-                        tt = ok ? tt : -INFINITY;
-                        st[nt][r] = tt;
-                        mx = fmaxf(mx, tt);
+                        if (win) { const int rel = j - qpos; ok = ok && rel < p.block_len && rel > -p.block_len; }
+                        st[nt][r] = ok ? st[nt][r] : -INFINITY;
                     }
-                mx = xhalf_max(mx);
-                m_new = fmaxf(m_run, mx);
+            }
+
+            // ---- running max: st already holds (score - m_run)
+            float mx = st[0][0];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[nt][r]);
+            mx = xhalf_max(mx);
+            const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
+            if (__any(raise)) {
+                const float delta = raise ? mx : 0.f;
+                const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
+                m_run += delta;
+                started = started || raise;
+                l_run *= scale;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float e = __builtin_amdgcn_exp2f(st[nt][r] - m_new);
-                        st[nt][r] = e;
-                        rsum += e;
-                    }
-            }
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            l_run = l_run * alpha + rsum;
-            if (__any(alpha != 1.0f)) {
+                    for (int r = 0; r < 16; ++r) st[nt][r] -= delta;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) ot[dt][r] *= scale;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
             }
 
-            // ---- O^T += V^T P^T
+            // ---- P = exp2(S^T);  O^T += V^T P^T
             const T* vs = Vs + buf * V_TILE;
             if constexpr (F32) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
+                        const float e = __builtin_amdgcn_exp2f(st[nt][r]);
+                        l_run += e;
                         // MFMA k-slot = lane half: half 0 feeds key 8g+t, half 1 key 8g+4+t
                         const int key = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt)
-                            ot[dt] = E::mfma(vs[key * VROWS + 32 * dt + lr], st[nt][r], ot[dt]);
+                            ot[dt] = E::mfma(vs[key * VROWS + 32 * dt + lr], e, ot[dt]);
                     }
             } else {
 #pragma unroll
@@ -513,8 +594,9 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
                     for (int u = 0; u < 2; ++u) {
                         f32x8 pv;
 #pragma unroll
-                        for (int x = 0; x < 8; ++x) pv[x] = st[nt][8 * u + x];
+                        for (int x = 0; x < 8; ++x) pv[x] = __builtin_amdgcn_exp2f(st[nt][8 * u + x]);
                         const v8 pb = __builtin_convertvector(pv, v8);
+                        l_run = E::sum8(pb, l_run);
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt) {
                             const int d = 32 * dt + lr;
@@ -557,7 +639,8 @@ __global__ __launch_bounds__(NTHREADS) void fwd_kernel(const FwdParams p) {
 // ------------------------------------------------------------------------ launch
 template <typename T, int D, int MODE, bool CAUSAL>
 static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
-    const size_t lut_bytes = p.table != nullptr ? (size_t)(2 * p.bs.sat + 1) * sizeof(float) : sizeof(float);
+    const int sat = p.table != nullptr ? p.bs.sat : 0;
+    const size_t lut_bytes = (size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float);
     const size_t smem = Geometry<T, D>::kTileBytes + lut_bytes;
     auto kern = fwd_kernel<T, D, MODE, CAUSAL>;
     if (smem > 48 * 1024) {
