@@ -101,6 +101,9 @@ constexpr int NTHREADS = 256;
 constexpr int NT = BN / 32;  // 32-key blocks per tile
 constexpr int LUT_PAD = 8;   // saturated entries kept on the left of the distance LUT
 constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
+#ifndef OCC
+#define OCC 2
+#endif
 
 __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
     int out = 0, d;
@@ -154,6 +157,12 @@ struct Geometry {
     static constexpr int K_TILE = BN * KSTR;
     static constexpr int V_TILE = VROWS * BN;          // 16-bit: V^T (dim x key); fp32: V (key x VROWS)
     static constexpr size_t kTileBytes = (size_t)(2 * K_TILE + 2 * V_TILE) * sizeof(T);
+    // XOR swizzles of the 16-byte chunk index (16-bit types).  The LDS has 64 four-byte banks, so
+    // a 16-byte read is conflict free when 16 consecutive lanes (rows) cover one 256-byte bank line.
+    static constexpr int RPL = 128 / D > 1 ? 128 / D : 1;   // K rows per bank line
+    static __device__ __forceinline__ int kswz(int row) { return (row / RPL) % CH; }
+    // V^T rows are always 128 bytes (64 keys); the extra term spreads the transposing writes
+    static __device__ __forceinline__ int vswz(int d) { return ((d >> 1) & 7) ^ ((d >> 4) & 7); }
 };
 
 // floats per shifted copy of the distance LUT (host and device agree through this)
@@ -163,7 +172,7 @@ __host__ __device__ inline int lut_quads(int sat, bool causal) {
 }
 
 template <typename T, int D, int MODE, bool CAUSAL>
-__global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
     using v8 = typename E::v8;
@@ -358,6 +367,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
         sg = t >= seg_nt[0] ? 1 : 0;
         j0 = seg_start[sg] + (t - (sg ? seg_nt[0] : 0)) * BN;
     };
+    // V staging unit of a thread (16-bit types): 4 keys x 4 dims.  Lane bits are spread so that the
+    // transposed 8-byte LDS writes of 32 consecutive lanes fall into 32 different 8-byte bank groups.
+    auto v_unit = [&](int idx, int& dg, int& kg, int& rot) {
+        if constexpr (D >= 64 && !F32) {
+            const int kb = (idx >> 3) & 1, kgx = (idx >> 5) & 7;
+            dg = (idx & 7) | (((idx >> 4) & 1) << 3) | ((idx >> 8) << 4);
+            kg = ((kgx >> 1) << 2) | (kb << 1) | (kgx & 1);
+            rot = (idx >> 4) & 1;
+        } else {
+            dg = idx % (D / 4); kg = idx / (D / 4); rot = 0;
+        }
+    };
     auto load_tile = [&](int t) {
         int sg, j0; tile_of(t, sg, j0);
         const __amdgpu_buffer_rsrc_t krs = sg ? seg_krs[1] : seg_krs[0];
@@ -383,7 +404,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int u = 0; u < V_PER_T; ++u) {
                 const int idx = tid + u * NTHREADS;
-                const int dg = idx % (D / 4), kg = idx / (D / 4);
+                int dg, kg, rot; v_unit(idx, dg, kg, rot);
                 if (V_UNITS % NTHREADS == 0 || idx < V_UNITS) {
                     u32x2 r[4];
 #pragma unroll
@@ -422,12 +443,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
                 const int idx = tid + c * NTHREADS;
                 const int row = idx / CH, ch = idx % CH;
                 if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS)
-                    *reinterpret_cast<u32x4*>(ks + row * D + ((ch ^ (row & (SW - 1))) * 8)) = kreg[c];
+                    *reinterpret_cast<u32x4*>(ks + row * D + ((ch ^ G::kswz(row)) * 8)) = kreg[c];
             }
 #pragma unroll
             for (int u = 0; u < V_PER_T; ++u) {
                 const int idx = tid + u * NTHREADS;
-                const int dg = idx % (D / 4), kg = idx / (D / 4);
+                int dg, kg, rot; v_unit(idx, dg, kg, rot);
                 if (V_UNITS % NTHREADS == 0 || idx < V_UNITS) {
                     // 4 keys x 4 dims -> 4 dims x 4 keys.  Key slots 4..7 and 8..11 of every 16 are
                     // swapped so that a lane's eight P values line up with one 16-byte V^T read.
@@ -438,14 +459,44 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
                     y[1] = u32x2{(a[0] >> 16) | (a[2] & 0xffff0000u), (c2[0] >> 16) | (c2[2] & 0xffff0000u)};
                     y[2] = u32x2{(a[1] & 0xffffu) | (a[3] << 16), (c2[1] & 0xffffu) | (c2[3] << 16)};
                     y[3] = u32x2{(a[1] >> 16) | (a[3] & 0xffff0000u), (c2[1] >> 16) | (c2[3] & 0xffff0000u)};
+                    // half of the lanes take the dims in the order 1,0,3,2: even and odd rows
+                    // (different halves of the 64 banks) are written by the same instruction
+                    const bool sw = rot != 0;
+                    const u32x2 z[4] = {sw ? y[1] : y[0], sw ? y[0] : y[1], sw ? y[3] : y[2], sw ? y[2] : y[3]};
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const int d = 4 * dg + c;
-                        *reinterpret_cast<u32x2*>(vs + d * BN + (((pk >> 1) ^ (d & 7)) * 8) + (pk & 1) * 4) = y[c];
+                        const int d = 4 * dg + (c ^ rot);
+                        *reinterpret_cast<u32x2*>(vs + d * BN + (((pk >> 1) ^ G::vswz(d)) * 8) + (pk & 1) * 4) = z[c];
                     }
                 }
             }
         }
+    };
+
+    // ---------------------------------------------------------------- tile classes (wavefront-uniform)
+    struct TileClass { int sg, j0, side; bool skip, use_lut, need_mask; };
+    auto classify = [&](int t) {
+        TileClass c;
+        c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
+        if (t >= ntiles) return c;
+        tile_of(t, c.sg, c.j0);
+        const int kind = seg_kind[c.sg];
+        const bool win = seg_win[c.sg] != 0;
+        int qlo, qhi;
+        if (kind == 0) { qlo = iw0 + P; qhi = iw1 + P; }
+        else if (kind == 1) { qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
+        else { qlo = iw0 / p.aux; qhi = iw1 / p.aux; }
+        const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
+        c.skip = iw0 >= row_end;                              // wavefront without live rows
+        if (CAUSAL) c.skip = c.skip || rel_min > 0;           // every key is in the future of every row
+        if (win) c.skip = c.skip || (rel_max <= -p.block_len) || (rel_min >= p.block_len);
+        const bool left_sat = rel_max <= -sat && (!CAUSAL || rel_max <= 0);
+        const bool right_sat = !CAUSAL && rel_min >= sat;
+        c.use_lut = has_lut && !(left_sat || right_sat);
+        c.need_mask = c.j0 + BN > seg_end[c.sg];
+        if (win) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
+        c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
+        return c;
     };
 
     // ---------------------------------------------------------------- running state
@@ -457,10 +508,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
     float m_run = 0.f;       // running max (base-2 units), meaningful once `started`
     float l_run = 0.f;       // running sum over this lane's half of the keys
     bool started = false;    // a finite score has been seen for this row
-    f32x16 cm;               // accumulator input of tiles with a constant bias: cb - m_run in every slot
-    float cb_cur = 0.f;
+    // accumulator input of tiles with a constant bias: (constant - m_run) in all 16 slots.  It is
+    // rewritten in ONE place (end of an iteration) when the running max was raised or the tiles
+    // crossed to the other saturated side, so the common path carries no copies of it.
+    f32x16 cm;
+    TileClass tc = classify(0);
+    int side_cur = tc.side;
+    float cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) cm[r] = 0.f;
+    for (int r = 0; r < 16; ++r) cm[r] = cb_cur;
 
     if (ntiles > 0) { load_tile(0); store_tile(0); }
     __syncthreads();
@@ -468,72 +524,81 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
     for (int t = 0; t < ntiles; ++t) {
         const int buf = t & 1;
         if (t + 1 < ntiles) load_tile(t + 1);
+        bool refill = false;
 
-        int sg, j0; tile_of(t, sg, j0);
-        const int kind = seg_kind[sg];
-        const int s_end = seg_end[sg];
-        const bool win = seg_win[sg] != 0;
-        // query positions of this lane / this wavefront in the segment's bias geometry
-        int qpos, qlo, qhi;
-        if (kind == 0) { qpos = irow + P; qlo = iw0 + P; qhi = iw1 + P; }
-        else if (kind == 1) { qpos = irow % p.block_len + p.aux; qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
-        else { qpos = irow / p.aux; qlo = iw0 / p.aux; qhi = iw1 / p.aux; }
-        const int rel_min = j0 - qhi, rel_max = j0 + BN - 1 - qlo;
+        if (!tc.skip) {
+            const int j0 = tc.j0;
+            const int kind = seg_kind[tc.sg];
+            const int s_end = seg_end[tc.sg];
+            const bool win = seg_win[tc.sg] != 0;
+            int qpos;    // this lane's query position in the segment's bias geometry
+            if (kind == 0) qpos = irow + P;
+            else if (kind == 1) qpos = irow % p.block_len + p.aux;
+            else qpos = irow / p.aux;
 
-        bool skip = iw0 >= row_end;                      // wavefront without live rows
-        if (CAUSAL) skip = skip || rel_min > 0;          // every key is in the future of every row
-        if (win) skip = skip || (rel_max <= -p.block_len) || (rel_min >= p.block_len);
-
-        if (!skip) {
-            const bool left_sat = rel_max <= -sat && (!CAUSAL || rel_max <= 0);
-            const bool right_sat = !CAUSAL && rel_min >= sat;
-            const bool use_lut = has_lut && !(left_sat || right_sat);
-            bool need_mask = j0 + BN > s_end;
-            if (win) need_mask = need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
-
-            // ---- accumulator input: bias - running max
-            f32x16 st[NT];
-            if (use_lut) {
-                const int e0 = j0 + 4 * hh - qpos + padl;
-                const float* lb = lut + (e0 & 3) * qlen;
-                const int y0 = e0 >> 2;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
-                        const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
-                    }
-            } else {
-                const float cb = has_bias ? (left_sat ? c_neg : c_pos) : 0.f;
-                if (cb != cb_cur) {   // wavefront-uniform: the tile moved to the other side of the diagonal
-                    cb_cur = cb;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) cm[r] = cb - m_run;
-                }
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) st[nt] = cm;
-            }
-
-            // ---- S^T = K Q^T + C
+            // ---- S^T = K Q^T + C, with C = bias - running max
             const T* ks = Ks + buf * K_TILE;
+            f32x16 st[NT];
+            if constexpr (F32) {
+                if (tc.use_lut) {
+                    const int e0 = j0 + 4 * hh - qpos + padl;
+                    const float* lb = lut + (e0 & 3) * qlen;
+                    const int y0 = e0 >> 2;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const int row = 32 * nt + lr;
+                    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int s = 0; s < KS; ++s) {
-                    if constexpr (F32) {
-                        st[nt] = E::mfma(ks[row * KSTR + 2 * s + hh], qf[s], st[nt]);
-                    } else {
-                        const v8 a = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ (row & (SW - 1))) * 8));
-                        st[nt] = E::mfma(a, qf[s], st[nt]);
+                        for (int g = 0; g < 4; ++g) {
+                            const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
+                            const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
+                        }
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) st[nt] = cm;
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int row = 32 * nt + lr;
+#pragma unroll
+                    for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ks[row * KSTR + 2 * s + hh], qf[s], st[nt]);
+                }
+            } else {
+                v8 ka[NT][KS];   // all K fragments of the tile: the LDS reads are in flight together
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int row = 32 * nt + lr;
+#pragma unroll
+                    for (int s = 0; s < KS; ++s)
+                        ka[nt][s] = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ G::kswz(row)) * 8));
+                }
+                if (tc.use_lut) {
+                    const int e0 = j0 + 4 * hh - qpos + padl;
+                    const float* lb = lut + (e0 & 3) * qlen;
+                    const int y0 = e0 >> 2;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
+                            const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
+                        }
+#pragma unroll
+                        for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
+                    }
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        st[nt] = E::mfma(ka[nt][0], qf[0], cm);   // cm stays live: untied accumulator input
+#pragma unroll
+                        for (int s = 1; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
                     }
                 }
             }
 
-            if (need_mask) {   // keys past the end of the segment, or outside the window
+            if (tc.need_mask) {   // keys past the end of the segment, or outside the window
                 const int jl = j0 + 4 * hh;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
@@ -555,6 +620,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
             mx = xhalf_max(mx);
             const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
             if (__any(raise)) {
+                asm volatile("");   // keep this rare block a real branch
                 const float delta = raise ? mx : 0.f;
                 const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
                 m_run += delta;
@@ -568,8 +634,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) ot[dt][r] *= scale;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
+                refill = true;
             }
 
             // ---- P = exp2(S^T);  O^T += V^T P^T
@@ -600,11 +665,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt) {
                             const int d = 32 * dt + lr;
-                            const v8 a = *reinterpret_cast<const v8*>(vs + d * BN + (((4 * nt + 2 * u + hh) ^ (d & 7)) * 8));
+                            const v8 a = *reinterpret_cast<const v8*>(vs + d * BN + (((4 * nt + 2 * u + hh) ^ G::vswz(d)) * 8));
                             ot[dt] = E::mfma(a, pb, ot[dt]);
                         }
                     }
             }
+        }
+
+        tc = classify(t + 1);
+        if (refill || (tc.side != 0 && tc.side != side_cur)) {
+            asm volatile("");
+            if (tc.side != 0) side_cur = tc.side;
+            cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
         }
 
         if (t + 1 < ntiles) store_tile(buf ^ 1);
