@@ -104,6 +104,11 @@ constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 #ifndef OCC
 #define OCC 2
 #endif
+#ifdef ABL_NOEXP
+#define ABL_EXP(x) (x)
+#else
+#define ABL_EXP(x) __builtin_amdgcn_exp2f(x)
+#endif
 
 __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
     int out = 0, d;
@@ -379,11 +384,10 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             dg = idx % (D / 4); kg = idx / (D / 4); rot = 0;
         }
     };
-    auto load_tile = [&](int t) {
+    auto load_tile_k = [&](int t) {
         int sg, j0; tile_of(t, sg, j0);
         const __amdgpu_buffer_rsrc_t krs = sg ? seg_krs[1] : seg_krs[0];
-        const __amdgpu_buffer_rsrc_t vrs = sg ? seg_vrs[1] : seg_vrs[0];
-        const int ksr = seg_ksr[sg], vsr = seg_vsr[sg];
+        const int ksr = seg_ksr[sg];
         // the whole byte offset goes into the vector operand: only that one is range checked
 #pragma unroll
         for (int c = 0; c < K_PER_T; ++c) {
@@ -392,6 +396,11 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS)
                 kreg[c] = __builtin_amdgcn_raw_buffer_load_b128(krs, (j0 + row) * ksr + ch * 16, 0, 0);
         }
+    };
+    auto load_tile_v = [&](int t) {
+        int sg, j0; tile_of(t, sg, j0);
+        const __amdgpu_buffer_rsrc_t vrs = sg ? seg_vrs[1] : seg_vrs[0];
+        const int vsr = seg_vsr[sg];
         if constexpr (F32) {
 #pragma unroll
             for (int c = 0; c < V_PER_T; ++c) {
@@ -416,20 +425,26 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             }
         }
     };
-    auto store_tile = [&](int buf) {
+    auto store_tile_k = [&](int buf) {
         T* ks = Ks + buf * K_TILE;
-        T* vs = Vs + buf * V_TILE;
-        if constexpr (F32) {
 #pragma unroll
-            for (int c = 0; c < K_PER_T; ++c) {
-                const int idx = tid + c * NTHREADS;
-                const int row = idx / CH, ch = idx % CH;
-                if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS) {
+        for (int c = 0; c < K_PER_T; ++c) {
+            const int idx = tid + c * NTHREADS;
+            const int row = idx / CH, ch = idx % CH;
+            if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS) {
+                if constexpr (F32) {
                     float* dst = reinterpret_cast<float*>(ks) + row * KSTR + ch * 4;
                     dst[0] = __uint_as_float(kreg[c][0]); dst[1] = __uint_as_float(kreg[c][1]);
                     dst[2] = __uint_as_float(kreg[c][2]); dst[3] = __uint_as_float(kreg[c][3]);
+                } else {
+                    *reinterpret_cast<u32x4*>(ks + row * D + ((ch ^ G::kswz(row)) * 8)) = kreg[c];
                 }
             }
+        }
+    };
+    auto store_tile_v = [&](int buf) {
+        T* vs = Vs + buf * V_TILE;
+        if constexpr (F32) {
 #pragma unroll
             for (int c = 0; c < V_PER_T; ++c) {
                 const int idx = tid + c * NTHREADS;
@@ -438,13 +453,6 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
                     *reinterpret_cast<u32x4*>(vs + row * VROWS + ch * 4) = vreg[c];
             }
         } else {
-#pragma unroll
-            for (int c = 0; c < K_PER_T; ++c) {
-                const int idx = tid + c * NTHREADS;
-                const int row = idx / CH, ch = idx % CH;
-                if (K_CHUNKS % NTHREADS == 0 || idx < K_CHUNKS)
-                    *reinterpret_cast<u32x4*>(ks + row * D + ((ch ^ G::kswz(row)) * 8)) = kreg[c];
-            }
 #pragma unroll
             for (int u = 0; u < V_PER_T; ++u) {
                 const int idx = tid + u * NTHREADS;
@@ -506,187 +514,231 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
     float m_run = 0.f;       // running max (base-2 units), meaningful once `started`
-    float l_run = 0.f;       // running sum over this lane's half of the keys
+    float l_run = 0.f;       // running sum over this lane's half of the keys (two partial sums)
+    float l_alt = 0.f;
     bool started = false;    // a finite score has been seen for this row
     // accumulator input of tiles with a constant bias: (constant - m_run) in all 16 slots.  It is
-    // rewritten in ONE place (end of an iteration) when the running max was raised or the tiles
-    // crossed to the other saturated side, so the common path carries no copies of it.
+    // rewritten in ONE place per step, when the running max was raised or the tiles crossed to
+    // the other saturated side, so the common path carries no copies of it.
     f32x16 cm;
-    TileClass tc = classify(0);
-    int side_cur = tc.side;
-    float cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
+    int side_cur = 0;
+    float cb_cur = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) cm[r] = cb_cur;
+    for (int r = 0; r < 16; ++r) cm[r] = 0.f;
 
-    if (ntiles > 0) { load_tile(0); store_tile(0); }
-    __syncthreads();
+    auto lane_qpos = [&](int sg) {   // this lane's query position in the segment's bias geometry
+        const int kind = seg_kind[sg];
+        if (kind == 0) return irow + P;
+        if (kind == 1) return irow % p.block_len + p.aux;
+        return irow / p.aux;
+    };
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) load_tile(t + 1);
-        bool refill = false;
-
-        if (!tc.skip) {
-            const int j0 = tc.j0;
-            const int kind = seg_kind[tc.sg];
-            const int s_end = seg_end[tc.sg];
-            const bool win = seg_win[tc.sg] != 0;
-            int qpos;    // this lane's query position in the segment's bias geometry
-            if (kind == 0) qpos = irow + P;
-            else if (kind == 1) qpos = irow % p.block_len + p.aux;
-            else qpos = irow / p.aux;
-
-            // ---- S^T = K Q^T + C, with C = bias - running max
+    // K fragments of one tile (16-bit types): issued early so that the LDS latency hides behind
+    // the softmax head of the previous tile
+    auto read_k = [&](int buf, v8 (&ka)[NT][KS]) {
+        if constexpr (!F32) {
             const T* ks = Ks + buf * K_TILE;
-            f32x16 st[NT];
-            if constexpr (F32) {
-                if (tc.use_lut) {
-                    const int e0 = j0 + 4 * hh - qpos + padl;
-                    const float* lb = lut + (e0 & 3) * qlen;
-                    const int y0 = e0 >> 2;
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt) {
+                const int row = 32 * nt + lr;
 #pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
-                            const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
-#pragma unroll
-                            for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
-                        }
-                } else {
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) st[nt] = cm;
-                }
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const int row = 32 * nt + lr;
-#pragma unroll
-                    for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ks[row * KSTR + 2 * s + hh], qf[s], st[nt]);
-                }
-            } else {
-                v8 ka[NT][KS];   // all K fragments of the tile: the LDS reads are in flight together
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const int row = 32 * nt + lr;
-#pragma unroll
-                    for (int s = 0; s < KS; ++s)
-                        ka[nt][s] = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ G::kswz(row)) * 8));
-                }
-                if (tc.use_lut) {
-                    const int e0 = j0 + 4 * hh - qpos + padl;
-                    const float* lb = lut + (e0 & 3) * qlen;
-                    const int y0 = e0 >> 2;
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
-                            const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
-#pragma unroll
-                            for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
-                        }
-#pragma unroll
-                        for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
-                    }
-                } else {
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        st[nt] = E::mfma(ka[nt][0], qf[0], cm);   // cm stays live: untied accumulator input
-#pragma unroll
-                        for (int s = 1; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
-                    }
-                }
+                for (int s = 0; s < KS; ++s)
+                    ka[nt][s] = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ G::kswz(row)) * 8));
             }
+        }
+    };
 
-            if (tc.need_mask) {   // keys past the end of the segment, or outside the window
-                const int jl = j0 + 4 * hh;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int j = jl + 32 * nt + 8 * (r >> 2) + (r & 3);
-                        bool ok = j < s_end;
-                        if (win) { const int rel = j - qpos; ok = ok && rel < p.block_len && rel > -p.block_len; }
-                        st[nt][r] = ok ? st[nt][r] : -INFINITY;
-                    }
-            }
-
-            // ---- running max: st already holds (score - m_run)
-            float mx = st[0][0];
+    // S^T = K Q^T + C for one tile, C = bias - running max (cm must be current for constant tiles)
+    auto compute_s = [&](const TileClass& c, int buf, const v8 (&ka)[NT][KS], f32x16 (&st)[NT]) {
+        const int qpos = lane_qpos(c.sg);
+        if (c.use_lut) {
+            const int e0 = c.j0 + 4 * hh - qpos + padl;
+            const float* lb = lut + (e0 & 3) * qlen;
+            const int y0 = e0 >> 2;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[nt][r]);
-            mx = xhalf_max(mx);
-            const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
-            if (__any(raise)) {
-                asm volatile("");   // keep this rare block a real branch
-                const float delta = raise ? mx : 0.f;
-                const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
-                m_run += delta;
-                started = started || raise;
-                l_run *= scale;
+                for (int g = 0; g < 4; ++g) {
+                    const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
+                    const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
+                    for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
+                }
+        }
+        if constexpr (F32) {
+            const T* ks = Ks + buf * K_TILE;
+            if (!c.use_lut) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) st[nt][r] -= delta;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) ot[dt][r] *= scale;
-                refill = true;
+                for (int nt = 0; nt < NT; ++nt) st[nt] = cm;
             }
-
-            // ---- P = exp2(S^T);  O^T += V^T P^T
-            const T* vs = Vs + buf * V_TILE;
-            if constexpr (F32) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int row = 32 * nt + lr;
+#pragma unroll
+                for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ks[row * KSTR + 2 * s + hh], qf[s], st[nt]);
+            }
+        } else {
+            if (c.use_lut) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const float e = __builtin_amdgcn_exp2f(st[nt][r]);
-                        l_run += e;
-                        // MFMA k-slot = lane half: half 0 feeds key 8g+t, half 1 key 8g+4+t
-                        const int key = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt)
-                            ot[dt] = E::mfma(vs[key * VROWS + 32 * dt + lr], e, ot[dt]);
-                    }
+                    for (int s = 0; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
             } else {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
+                for (int nt = 0; nt < NT; ++nt) {
+                    st[nt] = E::mfma(ka[nt][0], qf[0], cm);   // cm stays live: untied accumulator input
 #pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        f32x8 pv;
-#pragma unroll
-                        for (int x = 0; x < 8; ++x) pv[x] = __builtin_amdgcn_exp2f(st[nt][8 * u + x]);
-                        const v8 pb = __builtin_convertvector(pv, v8);
-                        l_run = E::sum8(pb, l_run);
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) {
-                            const int d = 32 * dt + lr;
-                            const v8 a = *reinterpret_cast<const v8*>(vs + d * BN + (((4 * nt + 2 * u + hh) ^ G::vswz(d)) * 8));
-                            ot[dt] = E::mfma(a, pb, ot[dt]);
-                        }
-                    }
+                    for (int s = 1; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
+                }
             }
         }
+    };
 
-        tc = classify(t + 1);
-        if (refill || (tc.side != 0 && tc.side != side_cur)) {
-            asm volatile("");
-            if (tc.side != 0) side_cur = tc.side;
-            cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
+    // mask, row max, lazy raise of the running max; returns true when m_run changed
+    auto softmax_head = [&](const TileClass& c, f32x16 (&st)[NT]) {
+        if (c.need_mask) {   // keys past the end of the segment, or outside the window
+            const int s_end = seg_end[c.sg];
+            const bool win = seg_win[c.sg] != 0;
+            const int qpos = lane_qpos(c.sg);
+            const int jl = c.j0 + 4 * hh;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int j = jl + 32 * nt + 8 * (r >> 2) + (r & 3);
+                    bool ok = j < s_end;
+                    if (win) { const int rel = j - qpos; ok = ok && rel < p.block_len && rel > -p.block_len; }
+                    st[nt][r] = ok ? st[nt][r] : -INFINITY;
+                }
         }
+        // st already holds (score - m_run)
+        float pm[4];   // four independent partial maxima: short dependency chains
+#pragma unroll
+        for (int c = 0; c < 4; ++c) pm[c] = st[0][4 * c];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) pm[c] = fmaxf(pm[c], st[nt][4 * c + x]);
+        float mx = xhalf_max(fmaxf(fmaxf(pm[0], pm[1]), fmaxf(pm[2], pm[3])));
+        const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
+        if (__any(raise)) {
+            asm volatile("");   // keep this rare block a real branch
+            const float delta = raise ? mx : 0.f;
+            const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
+            m_run += delta;
+            started = started || raise;
+            l_run *= scale;
+            l_alt *= scale;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) st[nt][r] -= delta;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ot[dt][r] *= scale;
+            return true;
+        }
+        return false;
+    };
 
-        if (t + 1 < ntiles) store_tile(buf ^ 1);
+    // P = exp2(S^T);  O^T += V^T P^T
+    auto compute_pv = [&](int buf, f32x16 (&st)[NT]) {
+        const T* vs = Vs + buf * V_TILE;
+        if constexpr (F32) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(st[nt][r]);
+                    l_run += e;
+                    // MFMA k-slot = lane half: half 0 feeds key 8g+t, half 1 key 8g+4+t
+                    const int key = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        ot[dt] = E::mfma(vs[key * VROWS + 32 * dt + lr], e, ot[dt]);
+                }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    f32x8 pv;
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) pv[x] = ABL_EXP(st[nt][8 * u + x]);
+                    const v8 pb = __builtin_convertvector(pv, v8);
+                    if (u == 0) l_run = E::sum8(pb, l_run); else l_alt = E::sum8(pb, l_alt);
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const int d = 32 * dt + lr;
+                        const v8 a = *reinterpret_cast<const v8*>(vs + d * BN + (((4 * nt + 2 * u + hh) ^ G::vswz(d)) * 8));
+                        ot[dt] = E::mfma(a, pb, ot[dt]);
+                    }
+                }
+        }
+    };
+
+    auto refill_cm = [&](int side) {
+        asm volatile("");
+        if (side != 0) side_cur = side;
+        cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
+    };
+
+    // ---------------------------------------------------------------- software pipeline
+    // Step t:   softmax head of tile t  ->  S MFMAs of tile t+1  ->  exp / PV MFMAs of tile t.
+    // The S product of the next tile is independent of the exp work of the current one, so the
+    // matrix pipe and the vector ALUs overlap inside one wavefront.  K tiles are staged two steps
+    // ahead and V tiles one step ahead, each in two LDS buffers, with one barrier per step.
+    f32x16 sta[NT], stb[NT];
+    TileClass tc = classify(0);
+    if (ntiles > 0) {
+        load_tile_k(0); load_tile_v(0);
+        store_tile_k(0); store_tile_v(0);
+        if (ntiles > 1) { load_tile_k(1); store_tile_k(1); }
+    }
+    __syncthreads();
+    if (tc.side != 0) refill_cm(tc.side);
+    if (ntiles > 0 && !tc.skip) {
+        v8 ka0[NT][KS];
+        read_k(0, ka0);
+        compute_s(tc, 0, ka0, sta);
+    }
+    __syncthreads();   // the first step overwrites the K buffer this product was read from
+
+    auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        const int buf = t & 1;
+#ifndef ABL_NOLOAD
+        if (t + 2 < ntiles) load_tile_k(t + 2);
+        if (t + 1 < ntiles) load_tile_v(t + 1);
+#endif
+        const TileClass nx = classify(t + 1);
+        v8 ka[NT][KS];
+        if (!nx.skip) read_k(buf ^ 1, ka);
+        bool refill = false;
+        if (!tc.skip) refill = softmax_head(tc, st);
+        if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        if (!nx.skip) compute_s(nx, buf ^ 1, ka, st_next);
+        if (!tc.skip) compute_pv(buf, st);
+#ifndef ABL_NOLOAD
+        if (t + 2 < ntiles) store_tile_k(buf);
+        if (t + 1 < ntiles) store_tile_v(buf ^ 1);
+#endif
+        tc = nx;
+#ifndef ABL_NOBAR
         __syncthreads();
+#endif
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        step(t, sta, stb);
+        if (t + 1 < ntiles) step(t + 1, stb, sta);
     }
 
     // ---------------------------------------------------------------- epilogue
-    const float l_tot = xhalf_sum(l_run);
+    const float l_tot = xhalf_sum(l_run + l_alt);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     if (row_ok && irow >= row_lo) {
         T* orow = op + (int64_t)irow * p.o_sr;
