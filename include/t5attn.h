@@ -134,7 +134,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           a ragged last block past L count as zero vectors (both as the
  *           reference computes them, attentions.py:722-732, :807-814).
  *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
- *           (B,H,n_side,D) projected block aggregates, bias bucket(g - i/aux).
+ *           (B,H,n_side,D) projected block aggregates, bias bucket(g - min(i/aux, n_side-1)).
  */
 typedef struct t5a_sparse_args {
     const void* q; const void* k; const void* v; void* o;

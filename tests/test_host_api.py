@@ -1,0 +1,144 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports what include/t5attn.h
+declares, argument validation works without a GPU, the host bucket table equals the oracle's, and
+the module surface mirrors the reference's."""
+import ctypes as C
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import t5_basic as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from turbot5_amd import _lib
+    return _lib
+
+
+def test_header_symbols_are_exported(lib):
+    header = open(os.path.join(ROOT, "include", "t5attn.h")).read()
+    declared = set(re.findall(r"\b(t5a_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(lib.EXPORTS)
+    handle = lib.load()
+    for name in declared:
+        assert getattr(handle, name) is not None
+    assert handle.t5a_version() >= 100
+
+
+def test_struct_sizes_follow_the_header(lib):
+    # natural alignment, no packing: catches a field added on one side only
+    assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8
+    assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 8 * 4 + C.sizeof(lib.T5ABias)
+    assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 2 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
+    assert C.sizeof(lib.T5ASparseArgs) == 6 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias)
+    assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4
+
+
+@pytest.mark.parametrize("bidirectional", [True, False])
+@pytest.mark.parametrize("nb,md", [(32, 128), (64, 256), (16, 64), (32, 20), (128, 512), (8, 1000), (256, 300)])
+def test_bucket_lut_equals_oracle(lib, bidirectional, nb, md):
+    got = lib.bucket_lut(bidirectional, nb, md)
+    rel = torch.arange(-md, md + 1)
+    want = O.relative_position_bucket(rel, bidirectional, nb, md).tolist()
+    assert got == want
+
+
+def test_bucket_lut_rejects_bad_parameters(lib):
+    for args in ((True, 2, 128), (False, 1, 128), (True, 32, 8), (True, 2048, 100000)):
+        with pytest.raises(lib.T5AError) as e:
+            lib.bucket_lut(*args)
+        assert e.value.code == -6
+
+
+def test_validation_without_gpu(lib):
+    handle = lib.load()
+    a = lib.T5ADenseArgs()
+    a.dtype, a.B, a.H, a.M, a.N, a.D = 0, 1, 1, 8, 8, 48
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -3          # head dim
+    assert b"head_dim" in handle.t5a_last_error()
+    a.D = 64
+    a.dtype = 7
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -2          # dtype
+    a.dtype = 0
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -1          # q is NULL
+    a.q = 0x1008
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -5          # misaligned
+    a.q = 0x1000
+    a.q_strides = (C.c_int64 * 3)(0, 0, 63)
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -5          # stride
+    assert handle.t5a_fwd_dense(None, None) == -1
+    a.M = -1
+    assert handle.t5a_fwd_dense(C.byref(a), None) == -4
+    a.M = 0
+    assert handle.t5a_fwd_dense(C.byref(a), None) == 0           # empty problem: nothing to launch
+    s = lib.T5ASparseArgs()
+    s.dtype, s.B, s.H, s.L, s.D, s.pattern, s.block_len = 0, 1, 1, 8, 64, 9, 4
+    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7
+    s.pattern, s.block_len, s.aux = 2, 4, 5
+    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7          # more global tokens than the block holds
+    k = lib.T5ASplitKArgs()
+    k.dtype, k.B, k.H, k.M, k.N, k.D, k.num_splits = 0, 1, 1, 1, 64, 64, 0
+    assert handle.t5a_fwd_splitk(C.byref(k), None) == -4
+    assert handle.t5a_splitk_workspace_bytes(2, 3, 1, 64, 4) == 2 * 3 * 4 * 1 * 66 * 4
+
+
+def test_ops_refuse_cpu_tensors():
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    q = torch.zeros(1, 1, 8, 64)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        flash_attention_with_fusing_bias(q, q, q, None)
+
+
+def test_function_signatures_match_the_reference():
+    """Names, order and defaults of fused_bias_attention.py:876 and varlen_fused_bias_attn.py:870."""
+    from turbot5_amd import ops
+    p = list(inspect.signature(ops.flash_attention_with_fusing_bias).parameters.items())[:8]
+    assert [(k, v.default) for k, v in p] == [
+        ("q", inspect._empty), ("k", inspect._empty), ("v", inspect._empty), ("bias", inspect._empty),
+        ("causal", False), ("sm_scale", None), ("NUM_BUCKETS", 32), ("MAX_DISTANCE", 128)]
+    p = list(inspect.signature(ops.flash_attention_with_fusing_bias_varlen).parameters.items())[:12]
+    assert [k for k, _ in p] == ["q", "k", "v", "bias", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q",
+                                 "max_seqlen_k", "causal", "sm_scale", "NUM_BUCKETS", "MAX_DISTANCE"]
+    assert [v.default for _, v in p][8:] == [False, None, 32, 128]
+    p = list(inspect.signature(ops.flash_attn_v2_fwd).parameters)
+    assert p == ["q", "k", "v", "bias", "causal", "sm_scale", "NUM_SPLITS", "BLOCK_M", "BLOCK_N", "num_warps",
+                 "num_stages"]
+
+
+def test_module_surface():
+    from turbot5_amd import T5ATTENTION_TYPES, T5Config, T5EncoderModel
+    assert {"flash", "local", "block", "transient-global"} <= set(T5ATTENTION_TYPES)
+    cfg = T5Config(d_model=64, d_kv=16, d_ff=128, num_layers=2, num_heads=4, vocab_size=50,
+                   attention_type="transient-global")
+    m = T5EncoderModel(cfg)
+    keys = set(m.state_dict())
+    p = "encoder.block.0.layer.0.SelfAttention."
+    for name in ("q.weight", "k.weight", "v.weight", "o.weight", "relative_attention_bias.weight",
+                 "global_relative_attention_bias.weight", "global_input_layer_norm.weight"):
+        assert p + name in keys
+    assert "encoder.block.1.layer.0.SelfAttention.relative_attention_bias.weight" not in keys
+    for name, cls in T5ATTENTION_TYPES.items():
+        sig = inspect.signature(cls.forward)
+        assert list(sig.parameters)[:3] == ["self", "hidden_states", "mask"]
+        assert "position_bias" in sig.parameters and "output_attentions" in sig.parameters
+    with pytest.raises(KeyError):
+        T5EncoderModel(cfg.copy(attention_type="full"))     # the reference's default is not a registry key either
+
+
+def test_padding_helpers_on_cpu():
+    from turbot5_amd.padding import _get_unpad_data, _upad_input, pad_input
+    mask = torch.tensor([[1, 1, 1, 0], [1, 0, 0, 0], [1, 1, 1, 1]])
+    idx, cu, mx = _get_unpad_data(mask)
+    idx2, cu2, _ = O.unpad_data(mask)
+    assert torch.equal(idx, idx2) and torch.equal(cu, cu2) and cu.dtype == torch.int32 and mx == 4
+    x = torch.arange(3 * 4 * 2 * 2, dtype=torch.float32).view(3, 4, 2, 2)
+    q, k, v, iq, (cq, ck), (mq, mk) = _upad_input(x, x, x, mask, 4, 2)
+    assert q.shape == (8, 2, 2) and torch.equal(cq, ck)
+    back = pad_input(q, iq, 3, 4)
+    assert torch.equal(back[mask.bool()], x[mask.bool()])
+    assert torch.equal(back[~mask.bool()], torch.zeros_like(back[~mask.bool()]))

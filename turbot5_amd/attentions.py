@@ -1,0 +1,321 @@
+"""Attention modules of the T5 encoder/decoder, drop-in for the reference's plugin classes.
+
+``T5ATTENTION_TYPES[config.attention_type](config, has_relative_attention_bias=...)`` builds the
+self-attention of an encoder layer exactly as the reference does
+(src/turbot5/model/modeling.py:54-61, :137).  Constructor and ``forward`` signatures, the
+returned tuple ``(attn_output, present_key_value, position_bias[, attn_weights])`` and the
+parameter names (``q k v o relative_attention_bias``, plus ``global_relative_attention_bias``
+and ``global_input_layer_norm`` for transient-global) are the reference's
+(src/turbot5/model/attentions.py:387-521, :523-649, :652-862, :865-1065), so HuggingFace T5 /
+LongT5 state dicts load unchanged.  The attention itself always runs in the HIP kernels of
+libt5attn.so; there is no torch fallback in this package.
+
+Differences from the reference, all on purpose:
+* every module hands the (num_buckets, H) TABLE on as ``position_bias`` (the reference does so
+  for 'flash' only; the sparse modules materialise a bias tensor), and never builds an L x L bias;
+* the sparse modules accept only all-ones attention masks (what ``T5Stack`` supplies when the
+  caller gives none); other masks raise ``NotImplementedError``;
+* transient-global returns the head-correct layout (the reference's ``unshape`` omits the
+  head transpose, attentions.py:951-953);
+* ``layer_head_mask`` and ``output_attentions`` are not available on fused paths.
+"""
+from __future__ import annotations
+
+import warnings
+from collections import OrderedDict
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import ops
+from .config import T5Config
+from .padding import _get_unpad_data, _upad_input, index_first_axis, pad_input
+
+
+class T5LayerNorm(nn.Module):
+    """RMS norm without mean subtraction or bias (reference src/turbot5/model/modules.py:24-67)."""
+
+    def __init__(self, dim: int, eps: float = 1e-6, use_triton: bool = False):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        variance = x.to(torch.float32).pow(2).mean(-1, keepdim=True)
+        x = x * torch.rsqrt(variance + self.eps)
+        if self.weight.dtype in (torch.float16, torch.bfloat16):
+            x = x.to(self.weight.dtype)
+        return self.weight * x
+
+
+# ---------------------------------------------------------------------------------------------
+# One host synchronisation per distinct mask tensor (not per layer): is it all ones, and if not,
+# where are the valid tokens.  The reference asks the same question in every layer
+# (attentions.py:410-418) and again inside the unpad helper (padding.py:82).
+_MASK_INFO: "OrderedDict[tuple, tuple]" = OrderedDict()
+
+
+def _mask_info(mask: torch.Tensor):
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), str(mask.device), mask.dtype)
+    hit = _MASK_INFO.get(key)
+    if hit is not None:
+        return hit
+    if mask.dim() != 2:
+        raise ValueError(f"attention mask must be (batch, key_length) of 0/1, got shape {tuple(mask.shape)}")
+    all_ones = bool((mask != 0).all())
+    unpad = None if all_ones else _get_unpad_data((mask != 0).to(torch.int32))
+    _MASK_INFO[key] = (all_ones, unpad)
+    while len(_MASK_INFO) > 16:
+        _MASK_INFO.popitem(last=False)
+    return all_ones, unpad
+
+
+class _T5AttentionBase(nn.Module):
+    """Parameters and shape helpers shared by the attention modules (attentions.py:36-66)."""
+
+    def __init__(self, config: T5Config, has_relative_attention_bias: bool = False):
+        super().__init__()
+        self.config = config
+        self.is_decoder = config.is_decoder
+        self.has_relative_attention_bias = has_relative_attention_bias
+        self.relative_attention_num_buckets = config.relative_attention_num_buckets
+        self.relative_attention_max_distance = config.relative_attention_max_distance
+        self.d_model = config.d_model
+        self.key_value_proj_dim = config.d_kv
+        self.n_heads = config.num_heads
+        self.dropout = config.dropout_rate
+        self.inner_dim = self.n_heads * self.key_value_proj_dim
+        self.q = nn.Linear(self.d_model, self.inner_dim, bias=False)
+        self.k = nn.Linear(self.d_model, self.inner_dim, bias=False)
+        self.v = nn.Linear(self.d_model, self.inner_dim, bias=False)
+        self.o = nn.Linear(self.inner_dim, self.d_model, bias=False)
+        if self.has_relative_attention_bias:
+            self.relative_attention_bias = nn.Embedding(self.relative_attention_num_buckets, self.n_heads)
+        self.pruned_heads = set()
+        self.gradient_checkpointing = False
+
+    # (B, L, H*D) -> strided (B, H, L, D) view; the kernels take the strides as they are
+    def _shape(self, states: torch.Tensor, batch_size: int) -> torch.Tensor:
+        return states.view(batch_size, -1, self.n_heads, self.key_value_proj_dim).transpose(1, 2)
+
+    def _unshape(self, states: torch.Tensor, batch_size: int) -> torch.Tensor:
+        return states.transpose(1, 2).contiguous().view(batch_size, -1, self.inner_dim)
+
+    def _attn_dtype(self, x: torch.Tensor) -> torch.dtype:
+        return self.config.attention_dtype or x.dtype
+
+    def _table(self, position_bias):
+        if position_bias is None and self.has_relative_attention_bias:
+            position_bias = self.relative_attention_bias.weight
+        if position_bias is not None and position_bias.dim() != 2:
+            raise ValueError("position_bias must be the (num_buckets, n_heads) table handed on by the first "
+                             f"layer, got shape {tuple(position_bias.shape)}")
+        return position_bias
+
+    @staticmethod
+    def _reject(layer_head_mask, output_attentions):
+        if layer_head_mask is not None:
+            raise NotImplementedError("layer_head_mask is not supported by the fused attention kernels")
+        if output_attentions:
+            raise NotImplementedError("attention weights are never materialised by the fused attention kernels")
+
+
+class T5FlashAttention(_T5AttentionBase):
+    """Full attention with the bias fused into the kernel (reference attentions.py:387-521).
+
+    Encoder self-attention (bidirectional buckets), decoder self-attention (``config.is_decoder``:
+    causal mask + unidirectional buckets, KV cache through ``past_key_value``) and cross-attention
+    (``cross_attention=True``: no causal mask; no bias unless a table is passed).
+    """
+
+    def __init__(self, config: T5Config, cross_attention: bool = False, *args, **kwargs) -> None:
+        super().__init__(config, *args, **kwargs)
+        self.causal = config.is_decoder and not cross_attention
+
+    def forward(self, hidden_states, mask=None, key_value_states=None, position_bias=None, past_key_value=None,
+                layer_head_mask=None, query_length=None, use_cache=False, output_attentions=False):
+        self._reject(layer_head_mask, output_attentions)
+        batch_size, seq_length = hidden_states.shape[:2]
+        varlen, unpad = False, None
+        if mask is not None:
+            all_ones, unpad = _mask_info(mask)
+            varlen = not all_ones
+
+        if past_key_value is not None and len(past_key_value) != 2:
+            raise ValueError(
+                f"past_key_value should have 2 past states: keys and values. Got { len(past_key_value)} past states")
+        adt = self._attn_dtype(hidden_states)
+
+        def project(proj_layer, past):
+            """keys or values: (B, H, key_length, D) in the attention dtype (attentions.py:444-469)."""
+            if key_value_states is None:
+                states = self._shape(proj_layer(hidden_states), batch_size).to(adt)
+                if past is not None:
+                    states = torch.cat([past, states], dim=2)
+                return states
+            if past is None or past.shape[2] != key_value_states.shape[1]:
+                return self._shape(proj_layer(key_value_states), batch_size).to(adt)
+            return past
+
+        query_states = self._shape(self.q(hidden_states), batch_size).to(adt)
+        key_states = project(self.k, past_key_value[0] if past_key_value is not None else None)
+        value_states = project(self.v, past_key_value[1] if past_key_value is not None else None)
+        table = self._table(position_bias)
+        nb, md = self.relative_attention_num_buckets, self.relative_attention_max_distance
+        key_length = key_states.shape[2]
+
+        if not varlen:
+            if table is None and not self.causal and seq_length <= 8 and key_length >= 512:
+                # few query rows over a long memory (incremental decoding): split-K kernel
+                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, 1.0)
+            else:
+                attn_output = ops.flash_attention_with_fusing_bias(
+                    query_states, key_states, value_states, table, causal=self.causal, sm_scale=1.0,
+                    NUM_BUCKETS=nb, MAX_DISTANCE=md)
+        else:
+            if mask.shape[1] != key_length:
+                raise ValueError(f"mask covers {mask.shape[1]} keys but there are {key_length}")
+            q_blhd = query_states.transpose(1, 2)
+            k_blhd = key_states.transpose(1, 2)
+            v_blhd = value_states.transpose(1, 2)
+            if key_value_states is None and seq_length == key_length:
+                q_p, k_p, v_p, indices_q, (cu_q, cu_k), (max_q, max_k) = _upad_input(
+                    q_blhd, k_blhd, v_blhd, mask, seq_length, self.n_heads, unpad_data=unpad)
+            else:
+                # queries are all valid; only the keys carry padding (cross-attention, cached decoding)
+                indices_k, cu_k, max_k = unpad
+                k_p = index_first_axis(k_blhd.reshape(batch_size * key_length, self.n_heads, -1), indices_k)
+                v_p = index_first_axis(v_blhd.reshape(batch_size * key_length, self.n_heads, -1), indices_k)
+                q_p = q_blhd.reshape(batch_size * seq_length, self.n_heads, -1)
+                cu_q = torch.arange(0, (batch_size + 1) * seq_length, seq_length, dtype=torch.int32,
+                                    device=hidden_states.device)
+                indices_q, max_q = None, seq_length
+            out_p = ops.flash_attention_with_fusing_bias_varlen(
+                q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
+                NUM_BUCKETS=nb, MAX_DISTANCE=md)
+            if indices_q is not None:
+                attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
+            else:
+                attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
+
+        attn_output = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
+        present_key_value_state = (key_states, value_states) if (self.is_decoder and use_cache) else None
+        return (attn_output,) + (present_key_value_state,) + (table,)
+
+
+class _SparseBase(_T5AttentionBase):
+    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions):
+        if past_key_value is not None:
+            warnings.warn('Currently, passing past key value states is not supported.')
+        if use_cache is not None:
+            warnings.warn('Currently, using cache is not supported for chosen attention type.')
+        self._reject(layer_head_mask, output_attentions)
+        if mask is not None:
+            all_ones, _ = _mask_info(mask)
+            if not all_ones:
+                raise NotImplementedError(
+                    f"{type(self).__name__} runs as tile skipping for all-ones attention masks only; "
+                    "use attention_type='flash' for padded batches")
+
+    def _qkv(self, hidden_states):
+        batch_size = hidden_states.shape[0]
+        adt = self._attn_dtype(hidden_states)
+        return tuple(self._shape(p(hidden_states), batch_size).to(adt) for p in (self.q, self.k, self.v))
+
+    def _finish(self, attn_output, hidden_states, table):
+        batch_size = hidden_states.shape[0]
+        out = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
+        return (out,) + (None,) + (table,)
+
+
+class T5LocalAttention(_SparseBase):
+    """Sliding-window attention, |j - i| < sliding_window (reference attentions.py:523-649)."""
+
+    def __init__(self, config: T5Config, *args, **kwargs) -> None:
+        super().__init__(config, *args, **kwargs)
+        self.block_len = config.sliding_window
+
+    def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
+                use_cache=None, output_attentions=False):
+        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        q, k, v = self._qkv(hidden_states)
+        table = self._table(position_bias)
+        # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
+        block_len = min(self.block_len, hidden_states.shape[1])
+        out = ops.local_attention_with_fusing_bias(
+            q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
+            self.relative_attention_max_distance)
+        return self._finish(out, hidden_states, table)
+
+
+class T5BlockAttention(_SparseBase):
+    """Own block plus ``global_block_size`` leading global tokens (reference attentions.py:652-862)."""
+
+    def __init__(self, config: T5Config, *args, **kwargs) -> None:
+        super().__init__(config, *args, **kwargs)
+        self.block_len = config.sliding_window
+        self.n_global_tokens = config.global_block_size
+
+    def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
+                use_cache=None, output_attentions=False):
+        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        q, k, v = self._qkv(hidden_states)
+        table = self._table(position_bias)
+        out = ops.block_attention_with_fusing_bias(
+            q, k, v, table, self.block_len, self.n_global_tokens, 1.0, self.relative_attention_num_buckets,
+            self.relative_attention_max_distance)
+        return self._finish(out, hidden_states, table)
+
+
+class T5TransientGlobalAttention(_SparseBase):
+    """Sliding window plus one side token per ``global_block_size`` tokens (reference attentions.py:865-1065)."""
+
+    def __init__(self, config: T5Config, *args, **kwargs) -> None:
+        super().__init__(config, *args, **kwargs)
+        self.block_len = config.sliding_window
+        self.global_block_size = config.global_block_size
+        if self.has_relative_attention_bias:
+            # kept for checkpoint compatibility; the reference reads the local table for the side
+            # bias as well (attentions.py:918-919)
+            self.global_relative_attention_bias = nn.Embedding(self.relative_attention_num_buckets, self.n_heads)
+        self.global_input_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+
+    def side_inputs(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """Normalised block sums, (B, L // global_block_size, d_model); trailing tokens that do not fill
+        a block join the last one (utils.py:206-212, :249-258; attentions.py:959-966)."""
+        B, L, d = hidden_states.shape
+        gbs = self.global_block_size
+        n_side = L // gbs
+        if n_side == 0:
+            return hidden_states.new_zeros(B, 0, d)
+        full = n_side * gbs
+        agg = hidden_states[:, :full].reshape(B, n_side, gbs, d).sum(dim=2)
+        if L > full:
+            agg = torch.cat([agg[:, :-1], agg[:, -1:] + hidden_states[:, full:].sum(dim=1, keepdim=True)], dim=1)
+        return self.global_input_layer_norm(agg)
+
+    def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
+                use_cache=None, output_attentions=False):
+        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        batch_size = hidden_states.shape[0]
+        adt = self._attn_dtype(hidden_states)
+        q, k, v = self._qkv(hidden_states)
+        side = self.side_inputs(hidden_states)
+        side_k = self._shape(self.k(side), batch_size).to(adt)
+        side_v = self._shape(self.v(side), batch_size).to(adt)
+        table = self._table(position_bias)
+        block_len = min(self.block_len, hidden_states.shape[1])
+        out = ops.transient_global_attention_with_fusing_bias(
+            q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
+            self.relative_attention_num_buckets, self.relative_attention_max_distance)
+        return self._finish(out, hidden_states, table)
+
+
+T5ATTENTION_TYPES = {
+    "flash": T5FlashAttention,
+    "triton-basic": T5FlashAttention,   # same math as 'flash'; the materialised-bias kernel is not rebuilt
+    "local": T5LocalAttention,
+    "block": T5BlockAttention,
+    "transient-global": T5TransientGlobalAttention,
+}

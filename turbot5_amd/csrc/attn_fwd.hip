@@ -493,7 +493,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         int qlo, qhi;
         if (kind == 0) { qlo = iw0 + P; qhi = iw1 + P; }
         else if (kind == 1) { qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
-        else { qlo = iw0 / p.aux; qhi = iw1 / p.aux; }
+        else { qlo = min(iw0 / p.aux, p.n_side - 1); qhi = min(iw1 / p.aux, p.n_side - 1); }
         const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
         c.skip = iw0 >= row_end;                              // wavefront without live rows
         if (CAUSAL) c.skip = c.skip || rel_min > 0;           // every key is in the future of every row
@@ -530,7 +530,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         const int kind = seg_kind[sg];
         if (kind == 0) return irow + P;
         if (kind == 1) return irow % p.block_len + p.aux;
-        return irow / p.aux;
+        return min(irow / p.aux, p.n_side - 1);   // trailing tokens past the last full block join it
     };
 
     // K fragments of one tile (16-bit types): issued early so that the LDS latency hides behind

@@ -1,0 +1,244 @@
+"""Lean T5 layer stack around the attention modules (the caller of the hot path).
+
+Restates the wiring of the reference's src/turbot5/model/modeling.py -- layer wrappers
+(:131-201), T5Block (:221-342), T5Stack (:352-632), T5EncoderModel (:834-942), T5Model (:635-831)
+-- without the HuggingFace ``PreTrainedModel`` machinery.  Parameter names equal HF T5's, so a
+T5 ``state_dict`` loads with ``load_state_dict``.  Differences from the reference:
+
+* every attention in the stack runs in the HIP kernels: the encoder uses
+  ``T5ATTENTION_TYPES[config.attention_type]``; the decoder self-attention is ``T5FlashAttention``
+  in causal mode with a KV cache, the cross-attention ``T5FlashAttention(cross_attention=True)``,
+  which switches to the split-K kernel for single-token steps (the reference keeps both on the
+  torch 'basic' path, modeling.py:134-135, :170);
+* layers receive the raw (batch, length) 0/1 mask (or None when the caller gives none) and the
+  (num_buckets, H) table of layer 0 as ``position_bias`` (modeling.py:589), never an L x L tensor.
+"""
+from __future__ import annotations
+
+import copy
+from typing import List, Optional, Tuple
+
+import torch
+from torch import nn
+
+from .attentions import T5ATTENTION_TYPES, T5FlashAttention, T5LayerNorm
+from .config import T5Config
+
+_ACT = {"relu": nn.functional.relu, "gelu": nn.functional.gelu, "silu": nn.functional.silu,
+        "gelu_new": lambda x: nn.functional.gelu(x, approximate="tanh")}
+
+
+class T5DenseActDense(nn.Module):
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.wi = nn.Linear(config.d_model, config.d_ff, bias=False)
+        self.wo = nn.Linear(config.d_ff, config.d_model, bias=False)
+        self.act = _ACT[config.dense_act_fn]
+
+    def forward(self, hidden_states):
+        return self.wo(self.act(self.wi(hidden_states)))
+
+
+class T5DenseGatedActDense(nn.Module):
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.wi_0 = nn.Linear(config.d_model, config.d_ff, bias=False)
+        self.wi_1 = nn.Linear(config.d_model, config.d_ff, bias=False)
+        self.wo = nn.Linear(config.d_ff, config.d_model, bias=False)
+        self.act = _ACT[config.dense_act_fn]
+
+    def forward(self, hidden_states):
+        return self.wo(self.act(self.wi_0(hidden_states)) * self.wi_1(hidden_states))
+
+
+class T5LayerFF(nn.Module):
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.DenseReluDense = T5DenseGatedActDense(config) if config.is_gated_act else T5DenseActDense(config)
+        self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+
+    def forward(self, hidden_states):
+        return hidden_states + self.DenseReluDense(self.layer_norm(hidden_states))
+
+
+class T5LayerSelfAttention(nn.Module):
+    def __init__(self, config: T5Config, has_relative_attention_bias=False):
+        super().__init__()
+        if config.is_decoder:
+            self.SelfAttention = T5FlashAttention(config, has_relative_attention_bias=has_relative_attention_bias)
+        else:
+            try:
+                cls = T5ATTENTION_TYPES[config.attention_type]
+            except KeyError:
+                raise KeyError(f"attention_type={config.attention_type!r}; available: {sorted(T5ATTENTION_TYPES)}") from None
+            self.SelfAttention = cls(config, has_relative_attention_bias=has_relative_attention_bias)
+        self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+
+    def forward(self, hidden_states, attention_mask=None, position_bias=None, layer_head_mask=None,
+                past_key_value=None, use_cache=False, output_attentions=False):
+        normed = self.layer_norm(hidden_states)
+        kwargs = dict(mask=attention_mask, position_bias=position_bias, layer_head_mask=layer_head_mask,
+                      past_key_value=past_key_value, output_attentions=output_attentions)
+        if isinstance(self.SelfAttention, T5FlashAttention):
+            kwargs["use_cache"] = use_cache
+        out = self.SelfAttention(normed, **kwargs)
+        return (hidden_states + out[0],) + out[1:]
+
+
+class T5LayerCrossAttention(nn.Module):
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.EncDecAttention = T5FlashAttention(config, cross_attention=True, has_relative_attention_bias=False)
+        self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+
+    def forward(self, hidden_states, key_value_states, attention_mask=None, position_bias=None,
+                past_key_value=None, use_cache=False, query_length=None):
+        normed = self.layer_norm(hidden_states)
+        out = self.EncDecAttention(normed, mask=attention_mask, key_value_states=key_value_states,
+                                   position_bias=position_bias, past_key_value=past_key_value,
+                                   use_cache=use_cache, query_length=query_length)
+        return (hidden_states + out[0],) + out[1:]
+
+
+class T5Block(nn.Module):
+    def __init__(self, config: T5Config, has_relative_attention_bias=False):
+        super().__init__()
+        self.is_decoder = config.is_decoder
+        self.layer = nn.ModuleList([T5LayerSelfAttention(config, has_relative_attention_bias)])
+        if self.is_decoder:
+            self.layer.append(T5LayerCrossAttention(config))
+        self.layer.append(T5LayerFF(config))
+
+    def forward(self, hidden_states, attention_mask=None, position_bias=None, encoder_hidden_states=None,
+                encoder_attention_mask=None, past_key_value=None, use_cache=False):
+        self_past = past_key_value[:2] if past_key_value is not None else None
+        cross_past = past_key_value[2:] if past_key_value is not None and len(past_key_value) == 4 else None
+        sa = self.layer[0](hidden_states, attention_mask=attention_mask, position_bias=position_bias,
+                           past_key_value=self_past, use_cache=use_cache)
+        hidden_states, present, position_bias = sa[0], sa[1], sa[2]
+        if self.is_decoder and encoder_hidden_states is not None:
+            ca = self.layer[1](hidden_states, key_value_states=encoder_hidden_states,
+                               attention_mask=encoder_attention_mask, past_key_value=cross_past,
+                               use_cache=use_cache)
+            hidden_states = ca[0]
+            if present is not None and ca[1] is not None:
+                present = present + ca[1]
+        hidden_states = self.layer[-1](hidden_states)
+        return hidden_states, present, position_bias
+
+
+class T5Stack(nn.Module):
+    def __init__(self, config: T5Config, embed_tokens: Optional[nn.Embedding] = None):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = embed_tokens
+        self.is_decoder = config.is_decoder
+        n = config.num_decoder_layers if config.is_decoder else config.num_layers
+        self.block = nn.ModuleList([T5Block(config, has_relative_attention_bias=bool(i == 0)) for i in range(n)])
+        self.final_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+
+    def forward(self, input_ids=None, attention_mask=None, encoder_hidden_states=None, encoder_attention_mask=None,
+                inputs_embeds=None, past_key_values=None, use_cache=False):
+        if inputs_embeds is None:
+            inputs_embeds = self.embed_tokens(input_ids)
+        hidden_states = inputs_embeds
+        if past_key_values is None:
+            past_key_values = [None] * len(self.block)
+        position_bias = None
+        presents: List[Optional[Tuple[torch.Tensor, ...]]] = []
+        # the decoder's own padding mask has no meaning under causal attention with right padding;
+        # only the encoder mask is routed down (as key padding of self- and cross-attention)
+        self_mask = None if self.is_decoder else attention_mask
+        for blk, past in zip(self.block, past_key_values):
+            hidden_states, present, position_bias = blk(
+                hidden_states, attention_mask=self_mask, position_bias=position_bias,
+                encoder_hidden_states=encoder_hidden_states, encoder_attention_mask=encoder_attention_mask,
+                past_key_value=past, use_cache=use_cache)
+            presents.append(present)
+        hidden_states = self.final_layer_norm(hidden_states)
+        return hidden_states, (presents if use_cache else None)
+
+
+def _init_t5_weights(module: nn.Module, config: T5Config) -> None:
+    """HuggingFace T5 initialisation scheme (the reference inherits it, modeling.py:344-350)."""
+    f = config.initializer_factor
+    d_model, d_kv, n_heads, d_ff = config.d_model, config.d_kv, config.num_heads, config.d_ff
+    for m in module.modules():
+        if isinstance(m, T5LayerNorm):
+            m.weight.data.fill_(f * 1.0)
+        elif isinstance(m, T5DenseActDense):
+            m.wi.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+            m.wo.weight.data.normal_(mean=0.0, std=f * (d_ff ** -0.5))
+        elif isinstance(m, T5DenseGatedActDense):
+            m.wi_0.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+            m.wi_1.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+            m.wo.weight.data.normal_(mean=0.0, std=f * (d_ff ** -0.5))
+        elif hasattr(m, "q") and hasattr(m, "o") and hasattr(m, "key_value_proj_dim"):
+            m.q.weight.data.normal_(mean=0.0, std=f * ((d_model * d_kv) ** -0.5))
+            m.k.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+            m.v.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+            m.o.weight.data.normal_(mean=0.0, std=f * ((n_heads * d_kv) ** -0.5))
+            if getattr(m, "has_relative_attention_bias", False):
+                m.relative_attention_bias.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+                if hasattr(m, "global_relative_attention_bias"):
+                    m.global_relative_attention_bias.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+
+
+class T5EncoderModel(nn.Module):
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.config = config
+        self.shared = nn.Embedding(config.vocab_size, config.d_model)
+        enc_cfg = config.copy(is_decoder=False, use_cache=False, is_encoder_decoder=False)
+        self.encoder = T5Stack(enc_cfg, self.shared)
+        self.shared.weight.data.normal_(mean=0.0, std=config.initializer_factor * 1.0)
+        _init_t5_weights(self, config)
+
+    def forward(self, input_ids=None, attention_mask=None, inputs_embeds=None):
+        return self.encoder(input_ids=input_ids, attention_mask=attention_mask, inputs_embeds=inputs_embeds)[0]
+
+
+class T5Model(nn.Module):
+    """Encoder-decoder with tied embeddings, an lm head and a greedy decoding loop."""
+
+    def __init__(self, config: T5Config):
+        super().__init__()
+        self.config = config
+        self.shared = nn.Embedding(config.vocab_size, config.d_model)
+        enc_cfg = config.copy(is_decoder=False, use_cache=False, is_encoder_decoder=False)
+        dec_cfg = config.copy(is_decoder=True, is_encoder_decoder=False)
+        self.encoder = T5Stack(enc_cfg, self.shared)
+        self.decoder = T5Stack(dec_cfg, self.shared)
+        self.lm_head = nn.Linear(config.d_model, config.vocab_size, bias=False)
+        self.shared.weight.data.normal_(mean=0.0, std=config.initializer_factor * 1.0)
+        self.lm_head.weight.data.normal_(mean=0.0, std=config.initializer_factor * 1.0)
+        _init_t5_weights(self, config)
+
+    def forward(self, input_ids, decoder_input_ids, attention_mask=None, encoder_outputs=None,
+                past_key_values=None, use_cache=False):
+        if encoder_outputs is None:
+            encoder_outputs = self.encoder(input_ids=input_ids, attention_mask=attention_mask)[0]
+        hidden, presents = self.decoder(input_ids=decoder_input_ids, encoder_hidden_states=encoder_outputs,
+                                        encoder_attention_mask=attention_mask, past_key_values=past_key_values,
+                                        use_cache=use_cache)
+        # tied embeddings are rescaled before the head, as T5 does (t5_heads.py: sequence_output * d_model**-0.5)
+        logits = self.lm_head(hidden * (self.config.d_model ** -0.5))
+        return logits, encoder_outputs, presents
+
+    @torch.no_grad()
+    def greedy_decode(self, input_ids=None, attention_mask=None, max_new_tokens: int = 16, encoder_outputs=None,
+                      batch_size: Optional[int] = None):
+        """Incremental greedy decoding: one token per step, self-attention over the KV cache through the
+        dense kernel, cross-attention over the encoder memory through the split-K kernel."""
+        if encoder_outputs is None:
+            encoder_outputs = self.encoder(input_ids=input_ids, attention_mask=attention_mask)[0]
+        B = encoder_outputs.shape[0] if batch_size is None else batch_size
+        dev = encoder_outputs.device
+        tokens = torch.full((B, 1), self.config.decoder_start_token_id, dtype=torch.long, device=dev)
+        out, past = [], None
+        for _ in range(max_new_tokens):
+            logits, _, past = self.forward(None, tokens, attention_mask=attention_mask,
+                                           encoder_outputs=encoder_outputs, past_key_values=past, use_cache=True)
+            tokens = logits[:, -1].argmax(dim=-1, keepdim=True)
+            out.append(tokens)
+        return torch.cat(out, dim=1)
