@@ -1,14 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-bias attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full] [--no-cpu] [--no-extra]
 
-A step is one launch of the dense fused-bias forward at the op-level T5-base shape
-(batch 16, 12 heads, head_dim 64, Lq = Lk = 1024, bf16, bidirectional buckets, no
-1/sqrt(d) scaling), inputs resident in HBM.  Prints ONE JSON line: the TFLOP/s of that
-workload (4*B*H*L*L*D algorithmic FLOPs per launch), the MFMA roofline fraction of the
-kernel measured with device events, a sweep over longer sequences, and the CPU 'basic'
-baseline timed on the host cores for a bounded sample of the same workload.
+A step is one launch of the dense fused-bias forward at the op-level T5-base shape (batch 16,
+12 heads, head_dim 64, Lq = Lk = 1024, bf16, bidirectional buckets, no 1/sqrt(d) scaling) with
+inputs resident in HBM.  Prints ONE JSON line:
+
+  value / ms_per_step   TFLOP/s of that workload (4*B*H*L*L*D algorithmic FLOPs per launch), wall
+                        clock around K launches with a device synchronise on both sides
+  roofline              the same kernel timed with device events on the launch stream, against the
+                        published dense bf16 MFMA peak
+  sweep                 longer sequences at constant B*L = 16384 (the "seq >= 4096" target)
+  extra                 the other workloads of the baseline: packed variable-length batch (bidirectional
+                        and causal), the three sparse patterns at L = 16384, T5-base encoder tokens/s at
+                        8k tokens; with --full also the 100k-token encoder pass and batch-64 greedy
+                        decoding over an 8192-token memory (split-K cross-attention)
+  cpu_baseline          the CPU 'basic' path (materialised bias, einsum, fp32 softmax, einsum) timed on
+                        the host cores on a bounded sample of the same workload
 """
 import argparse
 import json
@@ -21,6 +30,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 B, H, L, D = 16, 12, 1024, 64
 
 
@@ -48,9 +58,115 @@ def time_kernel(torch, fn, steps, warmup):
     return wall, dev_ms
 
 
+def c3_lengths(torch):
+    return torch.randint(128, 4097, (32,), generator=torch.Generator().manual_seed(1)).tolist()
+
+
+def extra_workloads(torch, dev, steps, full):
+    from turbot5_amd import ops
+    out = {}
+    reps, warm = max(5, steps // 5), 3
+
+    # ---- packed variable-length batch: 32 sequences, lengths U[128, 4096] (seed 1)
+    lens = c3_lengths(torch)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+    tot = sum(lens)
+    g = torch.Generator().manual_seed(3)
+    q, k, v = ((0.5 * torch.randn(tot, H, D, generator=g)).to(torch.bfloat16).to(dev) for _ in range(3))
+    table = torch.randn(32, H, generator=g).to(dev)
+    for causal in (False, True):
+        f = lambda: ops.flash_attention_with_fusing_bias_varlen(q, k, v, table, cu, cu, max(lens), max(lens),  # noqa: E731
+                                                                causal=causal, sm_scale=1.0)
+        _, ms = time_kernel(torch, f, reps, warm)
+        pairs = sum(n * (n + 1) // 2 for n in lens) if causal else sum(n * n for n in lens)
+        tf = 4.0 * H * D * pairs / (ms * 1e-3) / 1e12
+        out["varlen_causal" if causal else "varlen_bidirectional"] = {
+            "total_tokens": tot, "ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+    del q, k, v
+
+    # ---- sparse patterns, B1 H12 L16384 D64
+    Ls = 16384
+    q, k, v, table = make_inputs(torch, dev, 1, H, Ls, D, seed=4)
+    bytes_min = 4 * H * Ls * D * 2
+    f = lambda: ops.local_attention_with_fusing_bias(q, k, v, table, 128)  # noqa: E731
+    _, ms = time_kernel(torch, f, reps, warm)
+    pairs = Ls * 255 - 127 * 128
+    out["local_r127"] = {"ms": round(ms, 4), "tflops_live_pairs": round(4.0 * H * D * pairs / ms / 1e9, 1),
+                         "gbs_min_bytes": round(bytes_min / ms / 1e6, 1)}
+    f = lambda: ops.block_attention_with_fusing_bias(q, k, v, table, 128, 64)  # noqa: E731
+    _, ms = time_kernel(torch, f, reps, warm)
+    pairs = 64 * Ls + (Ls - 64) * 192 - 64 * 64
+    out["block_128_g64"] = {"ms": round(ms, 4), "tflops_live_pairs": round(4.0 * H * D * pairs / ms / 1e9, 1),
+                            "gbs_min_bytes": round(bytes_min / ms / 1e6, 1)}
+    g = torch.Generator().manual_seed(5)
+    sk, sv = ((0.5 * torch.randn(1, H, Ls // 16, D, generator=g)).to(torch.bfloat16).to(dev) for _ in range(2))
+    f = lambda: ops.transient_global_attention_with_fusing_bias(q, k, v, sk, sv, table, 128, 16)  # noqa: E731
+    _, ms = time_kernel(torch, f, reps, warm)
+    pairs = Ls * 255 - 127 * 128 + Ls * (Ls // 16)
+    out["tglobal_r127_g16"] = {"ms": round(ms, 4), "tflops_live_pairs": round(4.0 * H * D * pairs / ms / 1e9, 1)}
+    del q, k, v, sk, sv
+
+    # ---- T5-base encoder, tokens/s at 8k tokens
+    from turbot5_amd import T5Config, T5EncoderModel, T5Model
+    base = dict(vocab_size=32128, d_model=768, d_kv=64, d_ff=3072, num_layers=12, num_heads=12, dropout_rate=0.0,
+                attention_type="flash")
+    torch.manual_seed(0)
+    enc = T5EncoderModel(T5Config(attention_dtype=torch.bfloat16, **base)).eval().to(dev)
+    ids_g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        for bsz in (2, 1):
+            ids = torch.randint(0, 32128, (bsz, 8192), generator=ids_g).to(dev)
+            f = lambda: enc(ids)  # noqa: E731
+            _, ms = time_kernel(torch, f, 5, 2)
+            out[f"t5_base_encoder_8k_B{bsz}_fp32_act_bf16_attn"] = {
+                "ms": round(ms, 2), "tokens_per_s": round(bsz * 8192 / (ms * 1e-3), 1)}
+        enc16 = enc.to(torch.bfloat16)
+        enc16.config.attention_dtype = None
+        for blk in enc16.encoder.block:
+            blk.layer[0].SelfAttention.config.attention_dtype = None
+        ids = torch.randint(0, 32128, (2, 8192), generator=ids_g).to(dev)
+        f = lambda: enc16(ids)  # noqa: E731
+        _, ms = time_kernel(torch, f, 5, 2)
+        out["t5_base_encoder_8k_B2_bf16"] = {"ms": round(ms, 2), "tokens_per_s": round(2 * 8192 / (ms * 1e-3), 1)}
+        if full:
+            ids = torch.randint(0, 32128, (1, 100000), generator=ids_g).to(dev)
+            f = lambda: enc16(ids)  # noqa: E731
+            _, ms = time_kernel(torch, f, 2, 1)
+            attn_flops = 12 * 4.0 * 12 * 64 * 1e5 * 1e5
+            out["t5_base_encoder_100k_B1_bf16"] = {"ms": round(ms, 1), "tokens_per_s": round(1e5 / (ms * 1e-3), 1),
+                                                   "attention_tflops_lower_bound": round(attn_flops / ms / 1e9, 1)}
+    del enc
+    if full:
+        # ---- greedy decoding, batch 64 over an 8192-token encoder memory, 64 steps
+        torch.manual_seed(0)
+        model = T5Model(T5Config(attention_dtype=torch.bfloat16, **base)).eval().to(dev)
+        mem = torch.randn(64, 8192, 768, generator=torch.Generator().manual_seed(6)).to(dev)
+        steps_dec = 64
+        with torch.no_grad():
+            model.greedy_decode(encoder_outputs=mem, max_new_tokens=4)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            model.greedy_decode(encoder_outputs=mem, max_new_tokens=steps_dec)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        out["greedy_decode_B64_mem8192"] = {"steps": steps_dec, "ms_per_step": round(dt / steps_dec * 1e3, 3),
+                                            "tokens_per_s": round(64 * steps_dec / dt, 1)}
+        # the split-K cross-attention alone: one layer-step reads K and V of the whole memory once
+        g = torch.Generator().manual_seed(7)
+        kc = (0.5 * torch.randn(64, 8192, 12, 64, generator=g)).to(torch.bfloat16).to(dev).transpose(1, 2)
+        vc = (0.5 * torch.randn(64, 8192, 12, 64, generator=g)).to(torch.bfloat16).to(dev).transpose(1, 2)
+        qd = (0.5 * torch.randn(64, 12, 1, 64, generator=g)).to(torch.bfloat16).to(dev)
+        f = lambda: ops.flash_decoding_attention(qd, kc, vc, None, 1.0)  # noqa: E731
+        _, ms = time_kernel(torch, f, 20, 5)
+        nbytes = 2 * 64 * 8192 * 768 * 2
+        out["splitk_cross_attention_layer_step"] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                                                    "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    return out
+
+
 def cpu_baseline(torch, seconds_budget=20.0):
     """The oracle's 'basic' path (materialised bias, einsum, fp32 softmax, einsum) on the host cores,
-    on whole batch elements of the bench workload until ~the budget is used."""
+    on whole batch elements of the bench workload until about the budget is used."""
     from oracle import t5_basic as O
     threads = torch.get_num_threads()
     g = torch.Generator().manual_seed(0)
@@ -59,14 +175,14 @@ def cpu_baseline(torch, seconds_budget=20.0):
     O.dense_attention(q, k, v, table, False, 1.0)          # warm-up
     times = []
     t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < seconds_budget and len(times) < 16):
+    while len(times) < 3 or (time.perf_counter() - t_start < seconds_budget and len(times) < 64):
         t0 = time.perf_counter()
         O.dense_attention(q, k, v, table, False, 1.0)
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
     flops = 4.0 * H * L * L * D
-    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+    return {"value": round(flops / med / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"{len(times)} runs of 1 of the {B} batch elements (H{H} L{L} D{D}, fp32 'basic' with "
                       f"materialised bias), median {med * 1e3:.1f} ms"}
 
@@ -76,8 +192,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--full", action="store_true", help="also run the 100k-token encoder pass and the decode loop")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the longer-sequence sweep")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload (no sweep, no extra legs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -98,8 +215,8 @@ def main():
     value = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (dev_ms * 1e-3) / 1e12
 
-    sweep = {}
-    if not args.no_sweep:
+    sweep, extra = {}, {}
+    if not args.no_extra:
         for l in (2048, 4096, 8192, 16384):
             b = max(1, 16384 // l)
             qs, ks, vs, ts = make_inputs(torch, dev, b, H, l, D, seed=l)
@@ -108,6 +225,7 @@ def main():
             tf = 4.0 * b * H * l * l * D / (ms * 1e-3) / 1e12
             sweep[f"B{b}_L{l}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
             del qs, ks, vs, ts
+        extra = extra_workloads(torch, dev, args.steps, args.full)
 
     line = {
         "metric": "fused-bias attn fwd TFLOP/s + % MFMA peak; T5-base encoder tokens/s @8k",
@@ -119,10 +237,11 @@ def main():
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "kernel": "t5a::fwd_kernel<bf16,64,dense,false>", "kernel_ms": round(dev_ms, 5),
+                     "kernel": "t5a::fwd_kernel<bf16, 64, dense, non-causal>", "kernel_ms": round(dev_ms, 5),
                      "algorithmic_flops_per_launch": flops},
         "tokens_per_s": round(B * L / (wall_ms * 1e-3), 1),
         "sweep": sweep,
+        "extra": extra,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch)
