@@ -195,6 +195,8 @@ def main():
     ap.add_argument("--full", action="store_true", help="also run the 100k-token encoder pass and the decode loop")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload (no sweep, no extra legs)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run five plain 256 MiB device copies (calibrates the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -207,6 +209,14 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(dev)
+    if args.copy_probe:
+        x = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev)
+        y = torch.empty_like(x)
+        for _ in range(5):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes_per_copy": x.numel()}))
+        return
 
     q, k, v, table = make_inputs(torch, dev, B, H, L, D)
     fn = lambda: flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0)  # noqa: E731

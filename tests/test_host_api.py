@@ -142,3 +142,12 @@ def test_padding_helpers_on_cpu():
     back = pad_input(q, iq, 3, 4)
     assert torch.equal(back[mask.bool()], x[mask.bool()])
     assert torch.equal(back[~mask.bool()], torch.zeros_like(back[~mask.bool()]))
+
+
+def test_packed_workload_lengths_fixture():
+    import json
+    fx = json.load(open(os.path.join(ROOT, "tests", "golden", "c3_lengths.json")))
+    lens = torch.randint(128, 4097, (32,), generator=torch.Generator().manual_seed(1)).tolist()
+    assert fx["lengths"] == lens and fx["total"] == sum(lens)
+    import bench
+    assert bench.c3_lengths(torch) == lens
