@@ -161,13 +161,21 @@ struct Geometry {
     static constexpr int KSTR = F32 ? D + 1 : D;       // fp32 K rows padded by one float (bank spread)
     static constexpr int K_TILE = BN * KSTR;
     static constexpr int V_TILE = VROWS * BN;          // 16-bit: V^T (dim x key); fp32: V (key x VROWS)
-    static constexpr size_t kTileBytes = (size_t)(2 * K_TILE + 2 * V_TILE) * sizeof(T);
+    // 16-bit types with 128-byte rows are staged by LDS-DMA (buffer loads that write LDS directly):
+    // no staging registers, no vector ALU work, V stays row-major and is transposed on the LDS read.
+    static constexpr bool DMA = !F32 && D == 64;
+    static constexpr int NSK = DMA ? 4 : 2;             // LDS stages of K
+    static constexpr int NSV = DMA ? 4 : 2;             // LDS stages of V
+    static constexpr size_t kTileBytes = (size_t)(NSK * K_TILE + NSV * V_TILE) * sizeof(T);
     // XOR swizzles of the 16-byte chunk index (16-bit types).  The LDS has 64 four-byte banks, so
     // a 16-byte read is conflict free when 16 consecutive lanes (rows) cover one 256-byte bank line.
     static constexpr int RPL = 128 / D > 1 ? 128 / D : 1;   // K rows per bank line
     static __device__ __forceinline__ int kswz(int row) { return (row / RPL) % CH; }
     // V^T rows are always 128 bytes (64 keys); the extra term spreads the transposing writes
     static __device__ __forceinline__ int vswz(int d) { return ((d >> 1) & 7) ^ ((d >> 4) & 7); }
+    // row-major V (LDS-DMA path): the transposing read of a half wavefront touches 4 consecutive
+    // keys x 64 bytes; flipping the 64-byte halves of keys 2,3 (mod 4) spreads them over all banks
+    static __device__ __forceinline__ int vrow_swz(int key) { return ((key >> 1) & 1) << 2; }
 };
 
 // floats per shifted copy of the distance LUT (host and device agree through this)
@@ -189,9 +197,11 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     constexpr int ES = sizeof(T);
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T* Vs = reinterpret_cast<T*>(smem);         // [2][V_TILE]
-    T* Ks = Vs + 2 * V_TILE;                    // [2][K_TILE]
-    float* lut = reinterpret_cast<float*>(Ks + 2 * K_TILE);   // [4][4*quads]
+    constexpr bool DMA = G::DMA;
+    constexpr int NSK = G::NSK, NSV = G::NSV;
+    T* Vs = reinterpret_cast<T*>(smem);         // [NSV][V_TILE]
+    T* Ks = Vs + NSV * V_TILE;                  // [NSK][K_TILE]
+    float* lut = reinterpret_cast<float*>(Ks + NSK * K_TILE);   // [4][4*quads]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -332,7 +342,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         }
     }
     if (D < 32) {  // the part of V past head_dim feeds the MFMA: keep it zero
-        for (int idx = tid; idx < 2 * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
+        for (int idx = tid; idx < NSV * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
     }
     __syncthreads();
     const float c_neg = has_bias ? lut[0] : 0.f;                 // every key far before the query
@@ -382,6 +392,27 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             rot = (idx >> 4) & 1;
         } else {
             dg = idx % (D / 4); kg = idx / (D / 4); rot = 0;
+        }
+    };
+    // LDS-DMA staging: a wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses
+    // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
+    // physical chunk pc of row r fetches logical chunk pc ^ swizzle(r).  Rows past the end of the
+    // segment are out of the buffer's range and arrive as zeros.
+    auto dma_tile = [&](int t, bool is_v) {
+        if constexpr (DMA) {
+            int sg, j0; tile_of(t, sg, j0);
+            const __amdgpu_buffer_rsrc_t rs = is_v ? (sg ? seg_vrs[1] : seg_vrs[0]) : (sg ? seg_krs[1] : seg_krs[0]);
+            const int sr = is_v ? seg_vsr[sg] : seg_ksr[sg];
+            T* base = is_v ? Vs + (t % NSV) * V_TILE : Ks + (t % NSK) * K_TILE;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int slab = wave * 2 + c;              // 1 KB = 8 rows
+                const int r = slab * 8 + (lane >> 3), pc = lane & 7;
+                const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    rs, (__attribute__((address_space(3))) void*)(base + slab * 512), 16,
+                    (j0 + r) * sr + ch * 16, 0, 0, 0);
+            }
         }
     };
     auto load_tile_k = [&](int t) {
@@ -645,9 +676,42 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     };
 
     // P = exp2(S^T);  O^T += V^T P^T
+    // per-lane part of the transposing V reads (LDS-DMA path): within a group of 16 lanes, lane
+    // r = 4j + a supplies the address of V[key j][4a .. 4a+3] and receives, for head dim (lane % 16),
+    // the four keys j = 0..3 -- one 16 x 4 fragment of V^T per read, two reads per MFMA operand.
+    int vtr_off[2] = {0, 0};   // element offsets for dt = 0, 1 (before the per-block constants)
+    if constexpr (DMA) {
+        const int g = lane >> 4, r = lane & 15, jj = r >> 2, aa = r & 3;
+        const int row = 4 * (g >> 1) + jj;                      // + 32 nt + 16 u (+ 8 for the second read)
+        const int x = 2 * (g & 1) + (aa >> 1);
+        const int fb = G::vrow_swz(row) >> 2;                   // 0 or 1: swaps the 64-byte halves
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) vtr_off[dt] = row * D + ((4 * (dt ^ fb) + x) * 8) + (aa & 1) * 4;
+    }
     auto compute_pv = [&](int buf, f32x16 (&st)[NT]) {
         const T* vs = Vs + buf * V_TILE;
-        if constexpr (F32) {
+        if constexpr (DMA) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    f32x8 pv;
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) pv[x] = ABL_EXP(st[nt][8 * u + x]);
+                    const v8 pb = __builtin_convertvector(pv, v8);
+                    if (u == 0) l_run = E::sum8(pb, l_run); else l_alt = E::sum8(pb, l_alt);
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        typedef short s16x4 __attribute__((ext_vector_type(4)));
+                        typedef short s16x8 __attribute__((ext_vector_type(8)));
+                        const T* a0 = vs + vtr_off[dt] + (32 * nt + 16 * u) * D;
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
+                        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        ot[dt] = E::mfma(__builtin_bit_cast(v8, both), pb, ot[dt]);
+                    }
+                }
+        } else if constexpr (F32) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -693,9 +757,17 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     // The S product of the next tile is independent of the exp work of the current one, so the
     // matrix pipe and the vector ALUs overlap inside one wavefront.  K tiles are staged two steps
     // ahead and V tiles one step ahead, each in two LDS buffers, with one barrier per step.
+    //
+    // LDS-DMA path: K(t+4) and V(t+3) are requested in step t into four-stage rings; every step
+    // issues exactly four loads per wavefront (tiles past the end fetch zeros), so "at most eight
+    // loads outstanding" before the barrier means the tiles of the next step have landed.
     f32x16 sta[NT], stb[NT];
     TileClass tc = classify(0);
-    if (ntiles > 0) {
+    if constexpr (DMA) {
+        for (int i = 0; i < 4; ++i) dma_tile(i, false);
+        for (int i = 0; i < 3; ++i) dma_tile(i, true);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    } else if (ntiles > 0) {
         load_tile_k(0); load_tile_v(0);
         store_tile_k(0); store_tile_v(0);
         if (ntiles > 1) { load_tile_k(1); store_tile_k(1); }
@@ -710,27 +782,31 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     __syncthreads();   // the first step overwrites the K buffer this product was read from
 
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
-        const int buf = t & 1;
-#ifndef ABL_NOLOAD
-        if (t + 2 < ntiles) load_tile_k(t + 2);
-        if (t + 1 < ntiles) load_tile_v(t + 1);
-#endif
+        const int kbuf_next = DMA ? (t + 1) % NSK : (t + 1) & 1;
+        const int vbuf = DMA ? t % NSV : t & 1;
+        if constexpr (DMA) {
+            dma_tile(t + 4, false);
+            dma_tile(t + 3, true);
+        } else {
+            if (t + 2 < ntiles) load_tile_k(t + 2);
+            if (t + 1 < ntiles) load_tile_v(t + 1);
+        }
         const TileClass nx = classify(t + 1);
         v8 ka[NT][KS];
-        if (!nx.skip) read_k(buf ^ 1, ka);
+        if (!nx.skip) read_k(kbuf_next, ka);
         bool refill = false;
         if (!tc.skip) refill = softmax_head(tc, st);
         if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
-        if (!nx.skip) compute_s(nx, buf ^ 1, ka, st_next);
-        if (!tc.skip) compute_pv(buf, st);
-#ifndef ABL_NOLOAD
-        if (t + 2 < ntiles) store_tile_k(buf);
-        if (t + 1 < ntiles) store_tile_v(buf ^ 1);
-#endif
+        if (!nx.skip) compute_s(nx, kbuf_next, ka, st_next);
+        if (!tc.skip) compute_pv(vbuf, st);
+        if constexpr (DMA) {
+            __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8): everything but the last two steps' requests
+        } else {
+            if (t + 2 < ntiles) store_tile_k(t & 1);
+            if (t + 1 < ntiles) store_tile_v((t + 1) & 1);
+        }
         tc = nx;
-#ifndef ABL_NOBAR
         __syncthreads();
-#endif
     };
     for (int t = 0; t < ntiles; t += 2) {
         step(t, sta, stb);
