@@ -40,6 +40,8 @@
 //
 // Sparsity patterns are tile skipping: the key segments of a work item are
 // computed from integer positions; nothing outside them is loaded.
+#include <type_traits>
+
 #include "t5a_internal.h"
 
 namespace t5a {
@@ -138,6 +140,34 @@ __device__ __forceinline__ float xhalf_sum(float x) {
     const unsigned u = __float_as_uint(x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Raw buffer descriptor as four dwords (for the LDS-DMA loads issued from inline assembly)
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, unsigned bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+    // the descriptor is wavefront-uniform; say so, so that it lives in scalar registers
+    return u32x4{(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+                 (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu)),
+                 (unsigned)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+}
+
+// One LDS-DMA request: every lane fetches 16 bytes at its byte offset `voffset` of the buffer (zeros
+// when out of range) and the wavefront's 1 KB lands at LDS byte address `lds_addr` in lane order.
+// Issued from assembly so that the completion wait stays under the kernel's control: the step loop
+// waits with an explicit vmcnt(N) before its barrier instead of draining every request.
+__device__ __forceinline__ void lds_dma_16(u32x4 rs, unsigned lds_addr, int voffset) {
+    // descriptor and LDS address are wavefront-uniform; readfirstlane is free when the value already
+    // sits in scalar registers and makes the "s" constraints hold when the compiler kept it in vector ones
+    const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
+                        (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+}
+
+// barrier that orders LDS traffic only (lgkmcnt), leaving LDS-DMA requests in flight
+__device__ __forceinline__ void barrier_lds_only() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
@@ -314,12 +344,18 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     seg_nt[1] = nseg > 1 ? max(0, seg_end[1] - seg_start[1] + BN - 1) / BN : 0;
     const int ntiles = seg_nt[0] + seg_nt[1];
     __amdgpu_buffer_rsrc_t seg_krs[2], seg_vrs[2];
+    u32x4 seg_krw[2], seg_vrw[2];
 #pragma unroll
     for (int sg = 0; sg < 2; ++sg) {
         const int rows = min(seg_lend[sg], seg_end[sg]);   // rows at or past this read as zero
-        seg_krs[sg] = make_rsrc(seg_k[sg], rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_ksr[sg] + D * ES : 0u);
-        seg_vrs[sg] = make_rsrc(seg_v[sg], rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_vsr[sg] + D * ES : 0u);
+        const unsigned kb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_ksr[sg] + D * ES : 0u;
+        const unsigned vb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_vsr[sg] + D * ES : 0u;
+        seg_krs[sg] = make_rsrc(seg_k[sg], kb);
+        seg_vrs[sg] = make_rsrc(seg_v[sg], vb);
+        seg_krw[sg] = make_rsrc_words(seg_k[sg], kb);
+        seg_vrw[sg] = make_rsrc_words(seg_v[sg], vb);
     }
+    const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
     // ---------------------------------------------------------------- bias LUT
     const bool has_bias = p.table != nullptr;
@@ -398,20 +434,19 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
     // physical chunk pc of row r fetches logical chunk pc ^ swizzle(r).  Rows past the end of the
     // segment are out of the buffer's range and arrive as zeros.
-    auto dma_tile = [&](int t, bool is_v) {
+    auto dma_tile = [&](int t, bool is_v, int stage = -1) {
         if constexpr (DMA) {
             int sg, j0; tile_of(t, sg, j0);
-            const __amdgpu_buffer_rsrc_t rs = is_v ? (sg ? seg_vrs[1] : seg_vrs[0]) : (sg ? seg_krs[1] : seg_krs[0]);
+            const u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
             const int sr = is_v ? seg_vsr[sg] : seg_ksr[sg];
-            T* base = is_v ? Vs + (t % NSV) * V_TILE : Ks + (t % NSK) * K_TILE;
+            if (stage < 0) stage = is_v ? t % NSV : t % NSK;
+            const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
                 const int slab = wave * 2 + c;              // 1 KB = 8 rows
                 const int r = slab * 8 + (lane >> 3), pc = lane & 7;
                 const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rs, (__attribute__((address_space(3))) void*)(base + slab * 512), 16,
-                    (j0 + r) * sr + ch * 16, 0, 0, 0);
+                lds_dma_16(rs, base + slab * 1024, (j0 + r) * sr + ch * 16);
             }
         }
     };
@@ -574,7 +609,11 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
                 const int row = 32 * nt + lr;
 #pragma unroll
                 for (int s = 0; s < KS; ++s)
+#ifdef ABL_NOLDS
+                    ka[nt][s] = qf[(s + nt) % KS];
+#else
                     ka[nt][s] = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ G::kswz(row)) * 8));
+#endif
             }
         }
     };
@@ -708,7 +747,11 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
                         const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#ifdef ABL_NOLDS
+                        ot[dt] = E::mfma(qf[(dt + u) % KS], pb, ot[dt]);
+#else
                         ot[dt] = E::mfma(__builtin_bit_cast(v8, both), pb, ot[dt]);
+#endif
                     }
                 }
         } else if constexpr (F32) {
@@ -785,8 +828,10 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         const int kbuf_next = DMA ? (t + 1) % NSK : (t + 1) & 1;
         const int vbuf = DMA ? t % NSV : t & 1;
         if constexpr (DMA) {
+#ifndef ABL_NOLOAD
             dma_tile(t + 4, false);
             dma_tile(t + 3, true);
+#endif
         } else {
             if (t + 2 < ntiles) load_tile_k(t + 2);
             if (t + 1 < ntiles) load_tile_v(t + 1);
@@ -799,18 +844,67 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
         if (!nx.skip) compute_s(nx, kbuf_next, ka, st_next);
         if (!tc.skip) compute_pv(vbuf, st);
+        tc = nx;
         if constexpr (DMA) {
+#ifndef ABL_NOLOAD
             __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8): everything but the last two steps' requests
+#endif
+#ifndef ABL_NOBAR
+            barrier_lds_only();
+#endif
         } else {
             if (t + 2 < ntiles) store_tile_k(t & 1);
             if (t + 1 < ntiles) store_tile_v((t + 1) & 1);
+            __syncthreads();
         }
-        tc = nx;
-        __syncthreads();
     };
-    for (int t = 0; t < ntiles; t += 2) {
+    // Fast step (LDS-DMA path): tile t is a plain tile (no mask, not skipped) and tile t+1 is a
+    // plain constant-bias tile on the same side of the diagonal, so the step needs no tile
+    // classification and only one (rare) branch.  ST is the step index modulo 4, which fixes every
+    // LDS stage at compile time.
+    auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        constexpr int ST = decltype(st_c)::value;
+        dma_tile(t + 4, false, ST);
+        dma_tile(t + 3, true, (ST + 3) & 3);
+        v8 ka[NT][KS];
+        read_k((ST + 1) & 3, ka);
+        TileClass plain;
+        plain.sg = 0; plain.j0 = 0; plain.side = side_cur; plain.skip = false; plain.use_lut = false; plain.need_mask = false;
+        if (softmax_head(plain, st)) refill_cm(0);
+        compute_s(plain, (ST + 1) & 3, ka, st_next);
+        compute_pv(ST, st);
+        __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
+        barrier_lds_only();
+    };
+    // number of consecutive tiles from t on that are plain constant-bias tiles of one side
+    auto plain_run = [&](int t) {
+        int n = 0, side = -1;
+        for (; t + n < ntiles; ++n) {
+            const TileClass c = classify(t + n);
+            if (c.skip || c.need_mask || c.use_lut) break;
+            if (side < 0) side = c.side;
+            if (c.side != side) break;
+        }
+        return n;
+    };
+
+    int t = 0;
+    while (t < ntiles) {
+        if (DMA && (t & 3) == 0) {
+            // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5
+            int quads = (plain_run(t) - 1) >> 2;
+            for (; quads > 0; --quads, t += 4) {
+                fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
+                fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
+                fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
+                fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
+            }
+            if (t >= ntiles) break;
+            tc = classify(t);
+        }
         step(t, sta, stb);
         if (t + 1 < ntiles) step(t + 1, stb, sta);
+        t += 2;
     }
 
     // ---------------------------------------------------------------- epilogue
