@@ -106,6 +106,12 @@ constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 #ifndef OCC
 #define OCC 2
 #endif
+#ifndef T5A_PRIO
+#define T5A_PRIO 0
+#endif
+#ifndef T5A_SGB
+#define T5A_SGB 0
+#endif
 #ifdef ABL_NOEXP
 #define ABL_EXP(x) (x)
 #else
@@ -357,6 +363,36 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
+    auto tile_of = [&](int t, int& sg, int& j0) {
+        sg = t >= seg_nt[0] ? 1 : 0;
+        j0 = seg_start[sg] + (t - (sg ? seg_nt[0] : 0)) * BN;
+    };
+    // LDS-DMA staging: a wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses
+    // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
+    // physical chunk pc of row r fetches logical chunk pc ^ swizzle(r).  Rows past the end of the
+    // segment are out of the buffer's range and arrive as zeros.
+    auto dma_tile = [&](int t, bool is_v, int stage = -1) {
+        if constexpr (DMA) {
+            int sg, j0; tile_of(t, sg, j0);
+            const u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
+            const int sr = is_v ? seg_vsr[sg] : seg_ksr[sg];
+            if (stage < 0) stage = is_v ? t % NSV : t % NSK;
+            const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int slab = wave * 2 + c;              // 1 KB = 8 rows
+                const int r = slab * 8 + (lane >> 3), pc = lane & 7;
+                const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
+                lds_dma_16(rs, base + slab * 1024, (j0 + r) * sr + ch * 16);
+            }
+        }
+    };
+    // request the first tiles right away: they arrive while the bias LUT and the Q fragments are set up
+    if constexpr (DMA) {
+        for (int i = 0; i < 4; ++i) dma_tile(i, false);
+        for (int i = 0; i < 3; ++i) dma_tile(i, true);
+    }
+
     // ---------------------------------------------------------------- bias LUT
     const bool has_bias = p.table != nullptr;
     const bool has_lut = has_bias || CAUSAL;
@@ -414,10 +450,6 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     u32x4 kreg[K_PER_T];
     u32x4 vreg[F32 ? V_PER_T : 2 * V_PER_T];   // 16-bit: four 8-byte rows per unit
 
-    auto tile_of = [&](int t, int& sg, int& j0) {
-        sg = t >= seg_nt[0] ? 1 : 0;
-        j0 = seg_start[sg] + (t - (sg ? seg_nt[0] : 0)) * BN;
-    };
     // V staging unit of a thread (16-bit types): 4 keys x 4 dims.  Lane bits are spread so that the
     // transposed 8-byte LDS writes of 32 consecutive lanes fall into 32 different 8-byte bank groups.
     auto v_unit = [&](int idx, int& dg, int& kg, int& rot) {
@@ -428,26 +460,6 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             rot = (idx >> 4) & 1;
         } else {
             dg = idx % (D / 4); kg = idx / (D / 4); rot = 0;
-        }
-    };
-    // LDS-DMA staging: a wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses
-    // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
-    // physical chunk pc of row r fetches logical chunk pc ^ swizzle(r).  Rows past the end of the
-    // segment are out of the buffer's range and arrive as zeros.
-    auto dma_tile = [&](int t, bool is_v, int stage = -1) {
-        if constexpr (DMA) {
-            int sg, j0; tile_of(t, sg, j0);
-            const u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
-            const int sr = is_v ? seg_vsr[sg] : seg_ksr[sg];
-            if (stage < 0) stage = is_v ? t % NSV : t % NSK;
-            const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int slab = wave * 2 + c;              // 1 KB = 8 rows
-                const int r = slab * 8 + (lane >> 3), pc = lane & 7;
-                const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
-                lds_dma_16(rs, base + slab * 1024, (j0 + r) * sr + ch * 16);
-            }
         }
     };
     auto load_tile_k = [&](int t) {
@@ -549,10 +561,30 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
 
     // ---------------------------------------------------------------- tile classes (wavefront-uniform)
     struct TileClass { int sg, j0, side; bool skip, use_lut, need_mask; };
+    // dense / packed mode: one segment starting at key 0, so the class of tile t follows from four
+    // per-wavefront thresholds
+    int d_tl = 0, d_tr = 0, d_ts = 0, d_tm = 0;
+    if (MODE == kDense) {
+        const int qlo = iw0 + P, qhi = iw1 + P;
+        const int lim = qlo - (BN - 1) - sat;                  // left-saturated tiles: BN*t <= lim
+        d_tl = lim < 0 ? 0 : lim / BN + 1;
+        d_tr = CAUSAL ? 0x7fffffff : (qhi + sat <= 0 ? 0 : (qhi + sat + BN - 1) / BN);   // right-saturated from here
+        d_ts = iw0 >= row_end ? 0 : (CAUSAL ? (qhi < 0 ? 0 : qhi / BN + 1) : 0x7fffffff);  // skipped from here
+        d_tm = seg_end[0] / BN;                                // tiles from here on straddle the segment end
+    }
     auto classify = [&](int t) {
         TileClass c;
         c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
         if (t >= ntiles) return c;
+        if (MODE == kDense) {
+            c.j0 = t * BN;
+            c.skip = t >= d_ts;
+            const bool left_sat = t < d_tl, right_sat = t >= d_tr;
+            c.use_lut = has_lut && !(left_sat || right_sat);
+            c.need_mask = t >= d_tm;
+            c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
+            return c;
+        }
         tile_of(t, c.sg, c.j0);
         const int kind = seg_kind[c.sg];
         const bool win = seg_win[c.sg] != 0;
@@ -807,9 +839,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     f32x16 sta[NT], stb[NT];
     TileClass tc = classify(0);
     if constexpr (DMA) {
-        for (int i = 0; i < 4; ++i) dma_tile(i, false);
-        for (int i = 0; i < 3; ++i) dma_tile(i, true);
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the tiles requested at the top have landed
     } else if (ntiles > 0) {
         load_tile_k(0); load_tile_v(0);
         store_tile_k(0); store_tile_v(0);
@@ -858,32 +888,33 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             __syncthreads();
         }
     };
-    // Fast step (LDS-DMA path): tile t is a plain tile (no mask, not skipped) and tile t+1 is a
-    // plain constant-bias tile on the same side of the diagonal, so the step needs no tile
-    // classification and only one (rare) branch.  ST is the step index modulo 4, which fixes every
-    // LDS stage at compile time.
+    // Fast step (LDS-DMA path): tiles t and t+1 are neither skipped nor masked, so the step is the
+    // general one minus those cases.  ST is the step index modulo 4, which fixes every LDS stage at
+    // compile time.
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
         dma_tile(t + 4, false, ST);
         dma_tile(t + 3, true, (ST + 3) & 3);
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
-        TileClass plain;
-        plain.sg = 0; plain.j0 = 0; plain.side = side_cur; plain.skip = false; plain.use_lut = false; plain.need_mask = false;
-        if (softmax_head(plain, st)) refill_cm(0);
-        compute_s(plain, (ST + 1) & 3, ka, st_next);
+        TileClass cur;
+        cur.sg = tc.sg; cur.j0 = tc.j0; cur.side = 0; cur.skip = false; cur.use_lut = false; cur.need_mask = false;
+        const TileClass nx = classify(t + 1);
+        const bool refill = softmax_head(cur, st);
+        if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        compute_s(nx, (ST + 1) & 3, ka, st_next);
         compute_pv(ST, st);
+        tc = nx;
         __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
         barrier_lds_only();
     };
-    // number of consecutive tiles from t on that are plain constant-bias tiles of one side
+    // number of consecutive tiles from t on that are neither skipped nor masked
     auto plain_run = [&](int t) {
-        int n = 0, side = -1;
+        if (MODE == kDense) return max(0, min(min(d_ts, d_tm), ntiles) - t);
+        int n = 0;
         for (; t + n < ntiles; ++n) {
             const TileClass c = classify(t + n);
-            if (c.skip || c.need_mask || c.use_lut) break;
-            if (side < 0) side = c.side;
-            if (c.side != side) break;
+            if (c.skip || c.need_mask) break;
         }
         return n;
     };
@@ -893,6 +924,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         if (DMA && (t & 3) == 0) {
             // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5
             int quads = (plain_run(t) - 1) >> 2;
+            if (quads > 0) tc = classify(t);
             for (; quads > 0; --quads, t += 4) {
                 fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
                 fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
@@ -900,7 +932,6 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
                 fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
             }
             if (t >= ntiles) break;
-            tc = classify(t);
         }
         step(t, sta, stb);
         if (t + 1 < ntiles) step(t + 1, stb, sta);
