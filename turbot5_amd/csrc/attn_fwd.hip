@@ -40,6 +40,7 @@
 //
 // Sparsity patterns are tile skipping: the key segments of a work item are
 // computed from integer positions; nothing outside them is loaded.
+#include <atomic>
 #include <type_traits>
 
 #include "t5a_internal.h"
@@ -101,7 +102,10 @@ constexpr int BM = 128;      // query rows per workgroup
 constexpr int BN = 64;       // keys per tile
 constexpr int NTHREADS = 256;
 constexpr int NT = BN / 32;  // 32-key blocks per tile
-constexpr int LUT_PAD = 8;   // saturated entries kept on the left of the distance LUT
+// The distance LUT extends this far past the saturation distance on both sides.  A tile that takes
+// the LUT path has at least one unsaturated (row, key) pair, and a wavefront tile spans 32 rows x
+// 64 keys, so none of its distances lies more than 94 past saturation: lookups need no clamping.
+constexpr int LUT_PAD = 96;
 constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 #ifndef OCC
 #define OCC 2
@@ -216,8 +220,8 @@ struct Geometry {
 
 // floats per shifted copy of the distance LUT (host and device agree through this)
 __host__ __device__ inline int lut_quads(int sat, bool causal) {
-    const int e_right = sat + LUT_PAD + (causal ? 1 : sat);   // first index of the right-saturated part
-    return (e_right + 3) / 4 + 2;                              // quads 0 .. ymax, ymax = quads - 1
+    const int entries = sat + LUT_PAD + (causal ? 0 : sat) + LUT_PAD + 1;   // rel = -sat-PAD .. (sat|0)+PAD
+    return (entries + 3 + 3) / 4 + 1;                                      // + 3 for the shifted copies
 }
 
 template <typename T, int D, int MODE, bool CAUSAL>
@@ -393,6 +397,28 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         for (int i = 0; i < 3; ++i) dma_tile(i, true);
     }
 
+    // ---------------------------------------------------------------- Q fragments: loads first
+    const int iw0 = i0 + wave * 32;      // first row of this wavefront
+    const int iw1 = iw0 + 31;
+    const int irow = iw0 + lr;           // this lane's query row
+    const bool row_ok = irow < row_end;
+    v8 qf[KS];
+    f32x4 qraw[F32 ? D / 4 : 1];
+    if constexpr (F32) {
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            qraw[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (row_ok) qraw[c] = *reinterpret_cast<const f32x4*>(qp + (int64_t)irow * p.q_sr + 4 * c);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[s][e] = (T)0.0f;
+            if (row_ok) qf[s] = *reinterpret_cast<const v8*>(qp + (int64_t)irow * p.q_sr + 16 * s + 8 * hh);
+        }
+    }
+
     // ---------------------------------------------------------------- bias LUT
     const bool has_bias = p.table != nullptr;
     const bool has_lut = has_bias || CAUSAL;
@@ -402,15 +428,20 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     const int qlen = 4 * quads;
     const float log2e = 1.4426950408889634f;
     if (has_lut) {
-        for (int idx = tid; idx < 4 * qlen; idx += NTHREADS) {
-            const int a = idx / qlen, i = idx - a * qlen;
-            const int rel = i + a - padl;
+        // one evaluation per distance; the value goes to all four shifted copies:
+        // copy a, slot i holds the distance i + a - padl
+        for (int e = tid; e < qlen + 3; e += NTHREADS) {
+            const int rel = e - padl;
             float val = 0.f;
             if (has_bias)
                 val = load_table(p.table, p.table_dtype,
                                  (int64_t)bucket_of(p.bs, rel) * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
             if (CAUSAL && rel > 0) val = -INFINITY;
-            lut[idx] = val;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const int i = e - a;
+                if (i >= 0 && i < qlen) lut[a * qlen + i] = val;
+            }
         }
     }
     if (D < 32) {  // the part of V past head_dim feeds the MFMA: keep it zero
@@ -420,30 +451,18 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     const float c_neg = has_bias ? lut[0] : 0.f;                 // every key far before the query
     const float c_pos = has_bias ? lut[qlen - 1] : 0.f;          // every key far after it (non-causal)
 
-    // ---------------------------------------------------------------- Q fragments (pre-scaled)
-    const int iw0 = i0 + wave * 32;      // first row of this wavefront
-    const int iw1 = iw0 + 31;
-    const int irow = iw0 + lr;           // this lane's query row
-    const bool row_ok = irow < row_end;
-    v8 qf[KS];
+    // ---------------------------------------------------------------- Q fragments: pre-scale by sm_scale*log2(e)
     if constexpr (F32) {
 #pragma unroll
         for (int c = 0; c < D / 4; ++c) {
-            f32x4 x = {0.f, 0.f, 0.f, 0.f};
-            if (row_ok) x = *reinterpret_cast<const f32x4*>(qp + (int64_t)irow * p.q_sr + 4 * c);
-            qf[2 * c] = (hh ? x[1] : x[0]) * p.c1;
-            qf[2 * c + 1] = (hh ? x[3] : x[2]) * p.c1;
+            qf[2 * c] = (hh ? qraw[c][1] : qraw[c][0]) * p.c1;
+            qf[2 * c + 1] = (hh ? qraw[c][3] : qraw[c][2]) * p.c1;
         }
     } else {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            v8 x;
+        for (int s = 0; s < KS; ++s)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = (T)0.0f;
-            if (row_ok) x = *reinterpret_cast<const v8*>(qp + (int64_t)irow * p.q_sr + 16 * s + 8 * hh);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)x[e] * p.c1);
-        }
+            for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)qf[s][e] * p.c1);
     }
 
     // ---------------------------------------------------------------- tile staging
@@ -581,6 +600,9 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             c.skip = t >= d_ts;
             const bool left_sat = t < d_tl, right_sat = t >= d_tr;
             c.use_lut = has_lut && !(left_sat || right_sat);
+#ifdef ABL_NOLUTTILE
+            c.use_lut = false;
+#endif
             c.need_mask = t >= d_tm;
             c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
             return c;
@@ -626,9 +648,10 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
 
     auto lane_qpos = [&](int sg) {   // this lane's query position in the segment's bias geometry
         const int kind = seg_kind[sg];
-        if (kind == 0) return irow + P;
-        if (kind == 1) return irow % p.block_len + p.aux;
-        return min(irow / p.aux, p.n_side - 1);   // trailing tokens past the last full block join it
+        const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
+        if (kind == 0) return ir + P;
+        if (kind == 1) return ir % p.block_len + p.aux;
+        return min(ir / p.aux, p.n_side - 1);   // trailing tokens past the last full block join it
     };
 
     // K fragments of one tile (16-bit types): issued early so that the LDS latency hides behind
@@ -661,7 +684,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int y = min(max(y0 + 8 * nt + 2 * g, 0), quads - 1);
+                    const int y = y0 + 8 * nt + 2 * g;   // always inside the LUT, see LUT_PAD
                     const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
 #pragma unroll
                     for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
@@ -970,10 +993,12 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
     const size_t lut_bytes = (size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float);
     const size_t smem = Geometry<T, D>::kTileBytes + lut_bytes;
     auto kern = fwd_kernel<T, D, MODE, CAUSAL>;
-    if (smem > 48 * 1024) {
+    static std::atomic<size_t> granted{0};   // per instantiation: largest dynamic LDS size already allowed
+    if (smem > 48 * 1024 && smem > granted.load(std::memory_order_relaxed)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
+        granted.store(smem, std::memory_order_relaxed);
     }
     const unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NTHREADS), smem, stream, p);
