@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-bias attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full] [--no-cpu] [--no-extra] [--shape BxL[c]]
 
 A step is one launch of the dense fused-bias forward at the op-level T5-base shape (batch 16,
 12 heads, head_dim 64, Lq = Lk = 1024, bf16, bidirectional buckets, no 1/sqrt(d) scaling) with
@@ -31,6 +31,9 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+# HBM bytes per launch of the headline kernel: rocprofv3 FETCH_SIZE and WRITE_SIZE, each scaled by what the
+# same counter reads for a 256 MiB device copy (profiles/fwd_kernel_bf16_d64_dense_B16_L1024.hbm_traffic.txt)
+MEASURED_TRAFFIC_BYTES = 1.0103e8
 B, H, L, D = 16, 12, 1024, 64
 
 
@@ -42,20 +45,23 @@ def make_inputs(torch, dev, b, h, l, d, seed=0):
 
 
 def time_kernel(torch, fn, steps, warmup):
-    """(wall ms per step with host syncs on both sides, device-event ms per launch)."""
+    """(wall ms per step with host syncs on both sides, device ms per launch).
+
+    The device figure comes from one pair of events recorded on the launch stream (torch's current
+    stream, the one the library is handed) around the K back-to-back launches; events between the
+    launches would put marker packets into the queue and stretch the region they measure."""
     for _ in range(warmup):
         fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
-    for s, e in ev:
-        s.record()
+    start.record()
+    for _ in range(steps):
         fn()
-        e.record()
+    stop.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    dev_ms = sum(s.elapsed_time(e) for s, e in ev) / steps
-    return wall, dev_ms
+    return wall, start.elapsed_time(stop) / steps
 
 
 def c3_lengths(torch):
@@ -65,7 +71,7 @@ def c3_lengths(torch):
 def extra_workloads(torch, dev, steps, full):
     from turbot5_amd import ops
     out = {}
-    reps, warm = max(5, steps // 5), 3
+    reps, warm = max(10, steps // 2), 5
 
     # ---- packed variable-length batch: 32 sequences, lengths U[128, 4096] (seed 1)
     lens = c3_lengths(torch)
@@ -195,6 +201,8 @@ def main():
     ap.add_argument("--full", action="store_true", help="also run the 100k-token encoder pass and the decode loop")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload (no sweep, no extra legs)")
+    ap.add_argument("--shape", default=None, metavar="BxL[c]",
+                    help="only time the dense forward at batch B, length L (suffix c: causal); for profiling runs")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run five plain 256 MiB device copies (calibrates the HBM traffic counters)")
     args = ap.parse_args()
@@ -218,6 +226,17 @@ def main():
         print(json.dumps({"copy_probe_bytes_per_copy": x.numel()}))
         return
 
+    if args.shape:
+        causal = args.shape.endswith("c")
+        b, l = (int(x) for x in args.shape.rstrip("c").split("x"))
+        q, k, v, table = make_inputs(torch, dev, b, H, l, D, seed=l)
+        f = lambda: flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0)  # noqa: E731
+        _, ms = time_kernel(torch, f, args.steps, args.warmup)
+        fl = 4.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
+        print(json.dumps({"shape": args.shape, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
+                          "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}))
+        return
+
     q, k, v, table = make_inputs(torch, dev, B, H, L, D)
     fn = lambda: flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0)  # noqa: E731
     wall_ms, dev_ms = time_kernel(torch, fn, args.steps, args.warmup)
@@ -231,7 +250,7 @@ def main():
             b = max(1, 16384 // l)
             qs, ks, vs, ts = make_inputs(torch, dev, b, H, l, D, seed=l)
             f = lambda: flash_attention_with_fusing_bias(qs, ks, vs, ts, causal=False, sm_scale=1.0)  # noqa: E731
-            _, ms = time_kernel(torch, f, max(5, args.steps // 5), 3)
+            _, ms = time_kernel(torch, f, args.steps, args.warmup)
             tf = 4.0 * b * H * l * l * D / (ms * 1e-3) / 1e12
             sweep[f"B{b}_L{l}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
             del qs, ks, vs, ts
@@ -246,7 +265,7 @@ def main():
                                "32 buckets max_distance 128, sm_scale 1.0 (BASELINE config 2)",
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "t5a::fwd_kernel<bf16, 64, dense, non-causal>", "kernel_ms": round(dev_ms, 5),
                      "algorithmic_flops_per_launch": flops},
         "tokens_per_s": round(B * L / (wall_ms * 1e-3), 1),

@@ -76,6 +76,14 @@ def test_validation_without_gpu(lib):
     assert handle.t5a_fwd_dense(C.byref(a), None) == -4
     a.M = 0
     assert handle.t5a_fwd_dense(C.byref(a), None) == 0           # empty problem: nothing to launch
+    # one (batch, head) slice of K must stay below 2 GiB: 32-bit byte offsets inside the kernel
+    big = lib.T5ADenseArgs()
+    big.dtype, big.B, big.H, big.M, big.N, big.D = 0, 1, 1, 8, 1 << 20, 64
+    big.q = big.k = big.v = big.o = 0x1000
+    for name in ("q_strides", "k_strides", "v_strides", "o_strides"):
+        setattr(big, name, (C.c_int64 * 3)(0, 0, 2048))
+    assert handle.t5a_fwd_dense(C.byref(big), None) == -4
+    assert b"2 GiB" in handle.t5a_last_error()
     s = lib.T5ASparseArgs()
     s.dtype, s.B, s.H, s.L, s.D, s.pattern, s.block_len = 0, 1, 1, 8, 64, 9, 4
     assert handle.t5a_fwd_sparse(C.byref(s), None) == -7

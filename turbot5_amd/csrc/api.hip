@@ -108,6 +108,17 @@ static int check_tensor(const char* name, const void* ptr, const int64_t* stride
     return T5A_OK;
 }
 
+// The kernels address the key/value rows of one (batch, head) slice with 32-bit byte offsets and
+// prefetch a few tiles past the last row (those read as zeros): the slice must stay below 2 GiB.
+static int check_rows(const char* name, int64_t rows, int64_t row_stride, int dtype) {
+    const int64_t es = dtype == T5A_F32 ? 4 : 2;
+    if (row_stride < 0) return fail(T5A_ERR_STRIDE, "%s row stride %lld is negative", name, (long long)row_stride);
+    if ((rows + 1024) * row_stride * es > 0x7fffffffLL)
+        return fail(T5A_ERR_SHAPE, "%s: %lld rows of stride %lld elements exceed 2 GiB per (batch, head) slice", name,
+                    (long long)rows, (long long)row_stride);
+    return T5A_OK;
+}
+
 static int check_common(int dtype, int D) {
     if (dtype != T5A_BF16 && dtype != T5A_F16 && dtype != T5A_F32) return fail(T5A_ERR_DTYPE, "unsupported dtype %d", dtype);
     if (D != 16 && D != 32 && D != 64 && D != 128) return fail(T5A_ERR_HEAD_DIM, "head_dim %d not in {16,32,64,128}", D);
@@ -172,6 +183,8 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     if (a->N > 0) {
         if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
         if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
+        if ((rc = check_rows("k", a->N, a->k_strides[2], a->dtype))) return rc;
+        if ((rc = check_rows("v", a->N, a->v_strides[2], a->dtype))) return rc;
     }
     FwdParams p;
     memset(&p, 0, sizeof(p));
@@ -206,6 +219,8 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     if (a->total_k > 0) {
         if ((rc = check_tensor("k", a->k, a->k_strides, 2, unit))) return rc;
         if ((rc = check_tensor("v", a->v, a->v_strides, 2, unit))) return rc;
+        if ((rc = check_rows("k", a->max_seqlen_k, a->k_strides[0], a->dtype))) return rc;
+        if ((rc = check_rows("v", a->max_seqlen_k, a->v_strides[0], a->dtype))) return rc;
     }
     FwdParams p;
     memset(&p, 0, sizeof(p));
@@ -246,9 +261,13 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
     if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
     if ((rc = check_tensor("o", a->o, a->o_strides, 3, unit))) return rc;
+    if ((rc = check_rows("k", a->L, a->k_strides[2], a->dtype))) return rc;
+    if ((rc = check_rows("v", a->L, a->v_strides[2], a->dtype))) return rc;
     if (a->pattern == T5A_PATTERN_TGLOBAL && a->n_side > 0) {
         if ((rc = check_tensor("side_k", a->side_k, a->side_k_strides, 3, unit))) return rc;
         if ((rc = check_tensor("side_v", a->side_v, a->side_v_strides, 3, unit))) return rc;
+        if ((rc = check_rows("side_k", a->n_side, a->side_k_strides[2], a->dtype))) return rc;
+        if ((rc = check_rows("side_v", a->n_side, a->side_v_strides[2], a->dtype))) return rc;
     }
     FwdParams p;
     memset(&p, 0, sizeof(p));
