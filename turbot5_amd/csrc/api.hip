@@ -86,6 +86,7 @@ int make_bucket_spec(bool bidirectional, int num_buckets, int max_distance, Buck
     if (prev != s.nb - 1 || filled != s.n_thr)
         return fail(T5A_ERR_BUCKETS, "buckets do not saturate at max_distance=%d", max_distance);
     s.sat = s.n_thr > 0 ? s.thr[s.n_thr - 1] : s.max_exact;
+    for (int t = s.n_thr; t < kMaxThresholds; ++t) s.thr[t] = 0x7fffffff;   // unused slots never count
     if (s.sat > kMaxSaturation)
         return fail(T5A_ERR_BUCKETS, "bucket saturation distance %d exceeds %d", s.sat, kMaxSaturation);
     {

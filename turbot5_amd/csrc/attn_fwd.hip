@@ -127,8 +127,12 @@ __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
     if (s.bidirectional) { out = rel > 0 ? s.nb : 0; d = rel < 0 ? -rel : rel; }
     else { d = rel < 0 ? -rel : 0; }
     if (d < s.max_exact) return out + d;
+    // the first 16 thresholds come in with one scalar load and are compared without a loop
+    // (unused slots hold INT_MAX); the loop only runs for unusually fine bucketings
     int b = s.max_exact;
-    for (int t = 0; t < s.n_thr; ++t) b += (d >= s.thr[t]) ? 1 : 0;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) b += (d >= s.thr[t]) ? 1 : 0;
+    for (int t = 16; t < s.n_thr; ++t) b += (d >= s.thr[t]) ? 1 : 0;
     return out + b;
 }
 
@@ -141,10 +145,13 @@ __device__ __forceinline__ float load_table(const void* table, int dtype, int64_
 // max / sum over the two lanes (l, l^32) that share a query row; the swap
 // exchanges the upper half of one operand with the lower half of the other, so
 // combining both results is symmetric in the halves.
+// NaN-propagating maximum (v_maximum3_f32): unlike fmaxf it needs no quieting of its inputs, which
+// would cost one extra instruction per matrix-core result
+__device__ __forceinline__ float max_ieee(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 __device__ __forceinline__ float xhalf_max(float x) {
     const unsigned u = __float_as_uint(x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    return max_ieee(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float xhalf_sum(float x) {
     const unsigned u = __float_as_uint(x);
@@ -172,6 +179,17 @@ __device__ __forceinline__ void lds_dma_16(u32x4 rs, unsigned lds_addr, int voff
                         (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+}
+
+// Two requests that share one descriptor and one LDS base: the second carries an instruction offset of
+// 1024, which moves both its global and its LDS address (and takes part in the range check), so the
+// caller passes its lane offset minus 1024.
+__device__ __forceinline__ void lds_dma_16x2(unsigned lo, unsigned hi, unsigned bytes, unsigned lds_addr, int voff0, int voff1) {
+    const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)lo), (unsigned)__builtin_amdgcn_readfirstlane((int)hi),
+                        (unsigned)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
+                 "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory");
 }
 
 // barrier that orders LDS traffic only (lgkmcnt), leaving LDS-DMA requests in flight
@@ -355,6 +373,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     const int ntiles = seg_nt[0] + seg_nt[1];
     __amdgpu_buffer_rsrc_t seg_krs[2], seg_vrs[2];
     u32x4 seg_krw[2], seg_vrw[2];
+    int seg_kbytes0 = 0, seg_vbytes0 = 0;   // readable bytes of segment 0
 #pragma unroll
     for (int sg = 0; sg < 2; ++sg) {
         const int rows = min(seg_lend[sg], seg_end[sg]);   // rows at or past this read as zero
@@ -364,6 +383,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         seg_vrs[sg] = make_rsrc(seg_v[sg], vb);
         seg_krw[sg] = make_rsrc_words(seg_k[sg], kb);
         seg_vrw[sg] = make_rsrc_words(seg_v[sg], vb);
+        if (sg == 0) { seg_kbytes0 = (int)kb; seg_vbytes0 = (int)vb; }
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -389,6 +409,39 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
                 const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
                 lds_dma_16(rs, base + slab * 1024, (j0 + r) * sr + ch * 16);
             }
+        }
+    };
+    // Dense mode, fast steps: a running descriptor per tensor.  The tile's byte offset lives in the
+    // descriptor (base up, readable size down, clamped at zero so that tiles past the end still read
+    // zeros), advanced with a few scalar instructions per step, and the per-lane offsets are loop
+    // invariant.  Slices stay below 2 GiB (checked on the host), so signed 32-bit sizes do.
+    unsigned long long kcur = 0, vcur = 0;
+    int kleft = 0, vleft = 0;
+    const int kstep = BN * seg_ksr[0], vstep = BN * seg_vsr[0];
+    int cur_koff[2] = {0, 0}, cur_voff[2] = {0, 0};
+    if constexpr (DMA && MODE == kDense) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int r = (wave * 2 + c) * 8 + (lane >> 3), pc = lane & 7;
+            cur_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16 - c * 1024;
+            cur_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16 - c * 1024;
+        }
+    }
+    auto cursor_seek = [&](int tk, int tv) {   // next requests: K tile tk, V tile tv
+        kcur = reinterpret_cast<unsigned long long>(seg_k[0]) + (unsigned long long)((unsigned)tk * (unsigned)kstep);
+        vcur = reinterpret_cast<unsigned long long>(seg_v[0]) + (unsigned long long)((unsigned)tv * (unsigned)vstep);
+        kleft = seg_kbytes0 - tk * kstep;
+        vleft = seg_vbytes0 - tv * vstep;
+    };
+    auto cursor_dma = [&](int kstage, int vstage) {
+        if constexpr (DMA) {
+            const unsigned wbase = lds_base + (unsigned)wave * 2048u;
+            lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
+                         wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES, cur_koff[0], cur_koff[1]);
+            lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
+                         wbase + (unsigned)(vstage * V_TILE) * ES, cur_voff[0], cur_voff[1]);
+            kcur += (unsigned)kstep; vcur += (unsigned)vstep;
+            kleft -= kstep; vleft -= vstep;
         }
     };
     // request the first tiles right away: they arrive while the bias LUT and the Q fragments are set up
@@ -428,19 +481,32 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     const int qlen = 4 * quads;
     const float log2e = 1.4426950408889634f;
     if (has_lut) {
+        // The head's table column: with at most 64 buckets, lane b of every wavefront fetches bucket b
+        // up front (independent of the bucket arithmetic) and the LUT entries pick their value with a
+        // lane permute; larger tables are read per entry.
+        const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
+        const bool col_in_lanes = nbt <= 64;
+        float tcol = 0.f;
+        if (has_bias && col_in_lanes && lane < nbt)
+            tcol = load_table(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
         // one evaluation per distance; the value goes to all four shifted copies:
         // copy a, slot i holds the distance i + a - padl
-        for (int e = tid; e < qlen + 3; e += NTHREADS) {
+        for (int e0 = 0; e0 < qlen + 3; e0 += NTHREADS) {   // uniform trip count: the permute needs every lane
+            const int e = e0 + tid;
             const int rel = e - padl;
             float val = 0.f;
-            if (has_bias)
-                val = load_table(p.table, p.table_dtype,
-                                 (int64_t)bucket_of(p.bs, rel) * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+            if (has_bias) {
+                const int bk = bucket_of(p.bs, rel);
+                if (col_in_lanes)
+                    val = __int_as_float(__builtin_amdgcn_ds_bpermute(bk << 2, __float_as_int(tcol)));
+                else
+                    val = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+            }
             if (CAUSAL && rel > 0) val = -INFINITY;
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const int i = e - a;
-                if (i >= 0 && i < qlen) lut[a * qlen + i] = val;
+                if (i >= 0 && i < qlen && e < qlen + 3) lut[a * qlen + i] = val;
             }
         }
     }
@@ -745,8 +811,8 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int c = 0; c < 4; ++c)
 #pragma unroll
-                for (int x = 0; x < 4; ++x) pm[c] = fmaxf(pm[c], st[nt][4 * c + x]);
-        float mx = xhalf_max(fmaxf(fmaxf(pm[0], pm[1]), fmaxf(pm[2], pm[3])));
+                for (int x = 0; x < 4; ++x) pm[c] = max_ieee(pm[c], st[nt][4 * c + x]);
+        float mx = xhalf_max(max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3])));
         const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
         if (__any(raise)) {
             asm volatile("");   // keep this rare block a real branch
@@ -916,8 +982,8 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     // compile time.
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
-        dma_tile(t + 4, false, ST);
-        dma_tile(t + 3, true, (ST + 3) & 3);
+        if constexpr (MODE == kDense) cursor_dma(ST, (ST + 3) & 3);
+        else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
         TileClass cur;
@@ -925,6 +991,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         const TileClass nx = classify(t + 1);
         const bool refill = softmax_head(cur, st);
         if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): one wait for all K fragments instead of one per MFMA
         compute_s(nx, (ST + 1) & 3, ka, st_next);
         compute_pv(ST, st);
         tc = nx;
@@ -947,12 +1014,16 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         if (DMA && (t & 3) == 0) {
             // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5
             int quads = (plain_run(t) - 1) >> 2;
-            if (quads > 0) tc = classify(t);
-            for (; quads > 0; --quads, t += 4) {
+            if (quads > 0) {
+                tc = classify(t);
+                if constexpr (MODE == kDense) cursor_seek(t + 4, t + 3);
+            }
+            while (quads > 0) {
                 fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
                 fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
                 fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
                 fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
+                --quads; t += 4;
             }
             if (t >= ntiles) break;
         }
