@@ -1012,8 +1012,11 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     int t = 0;
     while (t < ntiles) {
         if (DMA && (t & 3) == 0) {
-            // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5
-            int quads = (plain_run(t) - 1) >> 2;
+            // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5.  When the run reaches the
+            // last tile, the final fast step forms an S product for a tile that does not exist (its K
+            // stage was filled with zeros) and nobody consumes it, so the run may end exactly there.
+            const int run = plain_run(t);
+            int quads = (t + run >= ntiles ? run : run - 1) >> 2;
             if (quads > 0) {
                 tc = classify(t);
                 if constexpr (MODE == kDense) cursor_seek(t + 4, t + 3);
