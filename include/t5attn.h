@@ -135,10 +135,15 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           reference computes them, attentions.py:722-732, :807-814).
  *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
  *           (B,H,n_side,D) projected block aggregates, bias bucket(g - min(i/aux, n_side-1)).
+ * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
+ * the G global rows, which attend all L keys, are computed as key splits spread over the whole
+ * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
+ * rounding of the merge.
  */
 typedef struct t5a_sparse_args {
     const void* q; const void* k; const void* v; void* o;
     const void* side_k; const void* side_v;
+    void* workspace; int64_t workspace_bytes;
     int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
     int64_t side_k_strides[3]; int64_t side_v_strides[3];
     int32_t dtype; int32_t B; int32_t H; int32_t L; int32_t D;
@@ -146,6 +151,7 @@ typedef struct t5a_sparse_args {
     float sm_scale; int32_t reserved;
     t5a_bias bias;
 } t5a_sparse_args;
+int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux);
 int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);
 
 /*

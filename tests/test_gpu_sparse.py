@@ -57,6 +57,29 @@ def test_block(gpu_device, dtype, L, Bl, G):
     assert (out.float().cpu() - want).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("L,Bl,G,D", [(2048, 128, 64, 64), (1900, 128, 33, 64), (4096, 256, 128, 32), (1536, 64, 16, 128)])
+def test_block_global_rows_as_key_splits(gpu_device, dtype, L, Bl, G, D):
+    """Long sequences: the G global rows are computed as key splits and merged (workspace given) or by one
+    workgroup per (batch, head) (no workspace); both against the oracle."""
+    from turbot5_amd.ops import block_attention_with_fusing_bias
+    from turbot5_amd import _lib
+    B, H = 2, 3
+    assert _lib.load().t5a_sparse_workspace_bytes(_lib.PATTERN_BLOCK, B, H, L, D, Bl, G) > 0
+    q, k, v = (rnd(B, H, L, D, seed=160 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=163, scale=1.0)
+    dev = [t.to(gpu_device) for t in (q, k, v, table)]
+    split = block_attention_with_fusing_bias(*dev, Bl, G)
+    single = block_attention_with_fusing_bias(*dev, Bl, G, key_splits=False)
+    if L % Bl == 0:
+        want = O.block_attention_blocked(q, k, v, table, Bl, G)
+        assert (split.float().cpu() - want).abs().max().item() <= TOL[dtype]
+        assert (single.float().cpu() - want).abs().max().item() <= TOL[dtype]
+    # the two ways differ only in the rounding of the merge, and only in the global rows
+    assert (split[:, :, :G].float() - single[:, :, :G].float()).abs().max().item() <= TOL[dtype]
+    assert torch.equal(split[:, :, G:], single[:, :, G:])
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("L,Bl,gbs", [(512, 128, 16), (256, 32, 8), (2048, 128, 16), (384, 64, 1)])
 def test_tglobal(gpu_device, dtype, L, Bl, gbs):

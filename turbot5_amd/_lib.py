@@ -17,7 +17,7 @@ PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
-    "t5a_fwd_sparse", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk",
+    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk",
 )
 
 
@@ -50,6 +50,7 @@ class T5AVarlenArgs(C.Structure):
 class T5ASparseArgs(C.Structure):
     _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
                 ("side_k", C.c_void_p), ("side_v", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
                 ("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3),
                 ("o_strides", C.c_int64 * 3), ("side_k_strides", C.c_int64 * 3), ("side_v_strides", C.c_int64 * 3),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("L", C.c_int32), ("D", C.c_int32),
@@ -101,6 +102,8 @@ def load() -> C.CDLL:
             fn.restype = C.c_int
         lib.t5a_splitk_workspace_bytes.argtypes = [C.c_int32] * 5
         lib.t5a_splitk_workspace_bytes.restype = C.c_int64
+        lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7
+        lib.t5a_sparse_workspace_bytes.restype = C.c_int64
         _lib = lib
     return _lib
 

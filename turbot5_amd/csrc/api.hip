@@ -244,6 +244,29 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
 }
 
+// Key splits for the global rows of the block pattern: enough (batch, head, split) items to fill the
+// device about twice, at least four key tiles of 64 per split.
+static void global_row_splits(int B, int H, int L, int* nsplit, int* split_rows) {
+    const int tiles = (L + 63) / 64;
+    const int64_t bh = (int64_t)B * H;
+    int64_t want = bh > 0 ? (512 + bh - 1) / bh : 1;
+    if (want > tiles / 4) want = tiles / 4;
+    if (want < 1) want = 1;
+    const int per = (int)((tiles + want - 1) / want);   // tiles per split
+    *split_rows = per * 64;
+    *nsplit = (tiles + per - 1) / per;
+}
+
+int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux) {
+    if (B < 0 || H < 0 || L < 0 || D < 0 || block_len <= 0 || aux < 0) return -1;
+    if (pattern != T5A_PATTERN_BLOCK || aux == 0 || L < block_len) return 0;
+    int nsplit, split_rows;
+    global_row_splits(B, H, L, &nsplit, &split_rows);
+    if (nsplit < 2) return 0;
+    const int64_t G = aux < L ? aux : L;
+    return (int64_t)B * H * nsplit * G * ((int64_t)D + 2) * (int64_t)sizeof(float);
+}
+
 int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
@@ -307,6 +330,29 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         g.tiles_per_seq = (g.M + 127) / 128;
         g.total_items = g.tiles_per_seq * a->H * a->B;
         g.align_end = 0;
+        const int64_t need = t5a_sparse_workspace_bytes(a->pattern, a->B, a->H, a->L, a->D, a->block_len, a->aux);
+        if (a->workspace != nullptr && need > 0) {
+            // key splits over the whole device, then one merge
+            if (a->workspace_bytes < need)
+                return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes, %lld needed", (long long)a->workspace_bytes, (long long)need);
+            if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+            global_row_splits(a->B, a->H, a->L, &g.nsplit, &g.split_rows);
+            const int64_t rows = (int64_t)a->B * a->H * g.nsplit * g.M;
+            g.part_o = reinterpret_cast<float*>(a->workspace);
+            g.part_l = g.part_o + rows * a->D;
+            g.part_m = g.part_l + rows;
+            const int64_t items = (int64_t)g.tiles_per_seq * g.nsplit * a->H * a->B;
+            if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
+            g.total_items = (int)items;
+            rc = finish(launch_fwd(g, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, global rows, key splits)");
+            if (rc) return rc;
+            SplitKParams m;
+            memset(&m, 0, sizeof(m));
+            m.o = a->o; m.part_o = g.part_o; m.part_l = g.part_l; m.part_m = g.part_m;
+            m.o_sb = p.o_sb; m.o_sh = p.o_sh; m.o_sr = p.o_sr;
+            m.B = a->B; m.H = a->H; m.M = g.M; m.S = g.nsplit;
+            return finish(launch_splitk_merge(m, a->dtype, a->D, s), "t5a_fwd_sparse(block, merge)");
+        }
         return finish(launch_fwd(g, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, global rows)");
     }
     p.tiles_per_seq = (a->L + 127) / 128;

@@ -275,7 +275,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (w >= p.total_items) return;
 
-    int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0;
+    int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     int64_t q_off, k_off, v_off, o_off, lse_off;
     if (MODE == kDense && p.cu_q != nullptr) {
         // packed batch: find (sequence, head, tile) by walking cu_seqlens
@@ -301,9 +301,10 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         v_off = (int64_t)ks * p.v_sr + (int64_t)h * p.v_sh;
         lse_off = (int64_t)qs * p.lse_sr + (int64_t)h * p.lse_sh;
     } else {
-        const int bh = w / p.tiles_per_seq;
+        int bh = w / p.tiles_per_seq;
         qt = w - bh * p.tiles_per_seq;
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
+        if (MODE == kDense && p.nsplit > 1) { split = bh % p.nsplit; bh /= p.nsplit; }
         b = bh / p.H;
         h = bh - b * p.H;
         Mseq = p.M;
@@ -313,6 +314,12 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
         v_off = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
         lse_off = (int64_t)b * p.lse_sb + (int64_t)h * p.lse_sh;
+        if (MODE == kDense && p.nsplit > 1) {   // this item sees only its slice of the keys
+            key0 = split * p.split_rows;
+            Nseq = max(0, min(p.split_rows, p.N - key0));
+            k_off += (int64_t)key0 * p.k_sr;
+            v_off += (int64_t)key0 * p.v_sr;
+        }
     }
     const T* qp = reinterpret_cast<const T*>(p.q) + q_off;
     T* op = reinterpret_cast<T*>(p.o) + o_off;
@@ -329,7 +336,7 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         i0 = qt * BM;
         row_end = Mseq;
     }
-    const int P = p.align_end ? Nseq - Mseq : 0;
+    const int P = p.align_end ? Nseq - Mseq : -key0;   // query position minus row index, in this item's key numbering
 
     // ---------------------------------------------------------------- key segments
     // A segment is a key range [start, end) of one K/V tensor.  Keys at or past
@@ -1038,7 +1045,29 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     // ---------------------------------------------------------------- epilogue
     const float l_tot = xhalf_sum(l_run + l_alt);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (row_ok && irow >= row_lo) {
+    if (MODE == kDense && p.nsplit > 1) {
+        // partial result of a key split: normalised row in fp32, weight 1 (0: no visible key) and log-sum-exp
+        if (row_ok) {
+            const int64_t prow = (((int64_t)b * p.H + h) * p.nsplit + split) * p.M + irow;
+            float* orow = p.part_o + prow * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d0 = 32 * dt + 8 * g + 4 * hh;
+                    if (d0 < D) {
+                        f32x4 x;
+#pragma unroll
+                        for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
+                        *reinterpret_cast<f32x4*>(orow + d0) = x;
+                    }
+                }
+            if (hh == 0) {
+                p.part_l[prow] = l_tot > 0.f ? 1.f : 0.f;
+                p.part_m[prow] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
+            }
+        }
+    } else if (row_ok && irow >= row_lo) {
         T* orow = op + (int64_t)irow * p.o_sr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)

@@ -200,6 +200,26 @@ static hipError_t launch_splitk_d(const SplitKParams& p, int D, hipStream_t s) {
     return hipErrorInvalidValue;
 }
 
+template <typename T>
+static hipError_t launch_merge_d(const SplitKParams& p, int D, hipStream_t s) {
+    const dim3 grid(p.M, p.H, p.B);
+    switch (D) {
+        case 16: hipLaunchKernelGGL((splitk_merge_kernel<T, 16>), grid, dim3(64), 0, s, p); break;
+        case 32: hipLaunchKernelGGL((splitk_merge_kernel<T, 32>), grid, dim3(64), 0, s, p); break;
+        case 64: hipLaunchKernelGGL((splitk_merge_kernel<T, 64>), grid, dim3(64), 0, s, p); break;
+        case 128: hipLaunchKernelGGL((splitk_merge_kernel<T, 128>), grid, dim3(128), 0, s, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_splitk_merge(const SplitKParams& p, int dtype, int D, hipStream_t stream) {
+    if (dtype == T5A_BF16) return launch_merge_d<__bf16>(p, D, stream);
+    if (dtype == T5A_F16) return launch_merge_d<_Float16>(p, D, stream);
+    if (dtype == T5A_F32) return launch_merge_d<float>(p, D, stream);
+    return hipErrorInvalidValue;
+}
+
 hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t stream) {
     if (dtype == T5A_BF16) return launch_splitk_d<__bf16>(p, D, stream);
     if (dtype == T5A_F16) return launch_splitk_d<_Float16>(p, D, stream);

@@ -42,6 +42,10 @@ struct FwdParams {
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;
     int block_len, aux, n_side;
     int align_end;       // 1: query i sits at key position i + N - M (KV-cache alignment); 0: at i
+    // key split (dense, unpacked, align_end == 0): split s of nsplit covers keys [s*split_rows, (s+1)*split_rows)
+    // and writes its normalised partial rows, a 1/0 weight and its log-sum-exp to the workspace arrays
+    int nsplit, split_rows;
+    float* part_o; float* part_l; float* part_m;   // (B,H,nsplit,M,D), (B,H,nsplit,M), (B,H,nsplit,M)
     BucketSpec bs;
 };
 
@@ -64,5 +68,7 @@ struct SplitKParams {
     float sm_scale;
 };
 hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t stream);
+// only the merge over splits (part_o, part_l, part_m -> o)
+hipError_t launch_splitk_merge(const SplitKParams& p, int dtype, int D, hipStream_t stream);
 
 }  // namespace t5a

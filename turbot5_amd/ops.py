@@ -149,7 +149,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
 
 
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
-            NUM_BUCKETS=32, MAX_DISTANCE=128):
+            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
     if k.shape != q.shape or v.shape != q.shape:
@@ -174,8 +174,14 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     a.pattern, a.block_len, a.aux = pattern, int(block_len), int(aux)
     a.sm_scale = float(sm_scale)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    lib = L.load()
+    ws_bytes = lib.t5a_sparse_workspace_bytes(pattern, B, H, Lq, D, int(block_len), int(aux))
+    workspace = None
+    if ws_bytes > 0 and key_splits:   # block pattern: key splits of the global rows
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = workspace.data_ptr(), ws_bytes
     with torch.cuda.device(q.device):
-        L.check(L.load().t5a_fwd_sparse(C.byref(a), _stream(q)))
+        L.check(lib.t5a_fwd_sparse(C.byref(a), _stream(q)))
     return o
 
 
@@ -188,11 +194,14 @@ def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM
 
 
 def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
-                                     MAX_DISTANCE=128):
+                                     MAX_DISTANCE=128, key_splits=True):
     """Block attention with ``n_global`` leading global tokens, the op of T5BlockAttention
-    (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout."""
+    (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout.
+
+    ``key_splits``: hand the library a workspace so that the global rows (which attend every key) are
+    spread over the device as key splits and merged; False keeps them in one workgroup per (batch, head)."""
     return _sparse(L.PATTERN_BLOCK, q, k, v, bias, block_len, n_global, None, None, sm_scale, NUM_BUCKETS,
-                   MAX_DISTANCE)
+                   MAX_DISTANCE, key_splits=key_splits)
 
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
