@@ -243,7 +243,7 @@ __host__ __device__ inline int lut_quads(int sat, bool causal) {
 }
 
 template <typename T, int D, int MODE, bool CAUSAL>
-__global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
     using v8 = typename E::v8;
@@ -301,12 +301,17 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
         v_off = (int64_t)ks * p.v_sr + (int64_t)h * p.v_sh;
         lse_off = (int64_t)qs * p.lse_sr + (int64_t)h * p.lse_sh;
     } else {
-        int bh = w / p.tiles_per_seq;
-        qt = w - bh * p.tiles_per_seq;
+        // unsigned arithmetic: the divisions are scalar code on every workgroup's critical path
+        unsigned bh = (unsigned)w / (unsigned)p.tiles_per_seq;
+        qt = (int)((unsigned)w - bh * (unsigned)p.tiles_per_seq);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
-        if (MODE == kDense && p.nsplit > 1) { split = bh % p.nsplit; bh /= p.nsplit; }
-        b = bh / p.H;
-        h = bh - b * p.H;
+        if (MODE == kDense && p.nsplit > 1) {
+            const unsigned g = bh / (unsigned)p.nsplit;
+            split = (int)(bh - g * (unsigned)p.nsplit);
+            bh = g;
+        }
+        b = (int)(bh / (unsigned)p.H);
+        h = (int)(bh - (unsigned)b * (unsigned)p.H);
         Mseq = p.M;
         Nseq = p.N;
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
@@ -453,8 +458,14 @@ __global__ __launch_bounds__(NTHREADS, OCC) void fwd_kernel(const FwdParams p) {
     };
     // request the first tiles right away: they arrive while the bias LUT and the Q fragments are set up
     if constexpr (DMA) {
-        for (int i = 0; i < 4; ++i) dma_tile(i, false);
-        for (int i = 0; i < 3; ++i) dma_tile(i, true);
+        if constexpr (MODE == kDense) {
+            cursor_seek(0, 0);
+            cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
+            dma_tile(3, false);                                     // K3
+        } else {
+            for (int i = 0; i < 4; ++i) dma_tile(i, false);
+            for (int i = 0; i < 3; ++i) dma_tile(i, true);
+        }
     }
 
     // ---------------------------------------------------------------- Q fragments: loads first
