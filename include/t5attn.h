@@ -177,6 +177,27 @@ typedef struct t5a_splitk_args {
 int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, int32_t num_splits);
 int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
 
+/*
+ * T5 RMS norm (no mean subtraction, no bias) and, with group > 1, the side-token producer of the
+ * transient-global pattern: output row r of a sequence is the norm of the SUM of input rows
+ * [r*group, (r+1)*group), the rows left over at the end of the sequence joining its last group.
+ * Replaces T5LayerNorm (src/turbot5/model/modules.py:24-67; Triton variant src/turbot5/ops/
+ * rms_norm.py:5-48) and, for group > 1, _create_global_aggregates + global_input_layer_norm
+ * (src/turbot5/model/utils.py:249-258, :206-212; src/turbot5/model/attentions.py:959-966), all-ones mask.
+ * x: (batches, rows_per_batch, dim) with strides {batch, row} in elements, dim contiguous and a
+ * multiple of 8; weight: (dim); y: (batches, rows_per_batch / group, dim) contiguous, in the
+ * weight's type when that is 16 bit, else fp32 (torch type promotion of the reference code).
+ * Arithmetic as the reference's eager path: fp32 variance and scaling, the scaled value rounded to
+ * a 16-bit weight's type before the product; block sums are rounded to the input type first.
+ */
+typedef struct t5a_rmsnorm_args {
+    const void* x; const void* weight; void* y;
+    int64_t x_strides[2];
+    int64_t batches; int32_t rows_per_batch; int32_t dim; int32_t group;
+    int32_t x_dtype; int32_t weight_dtype; float eps;
+} t5a_rmsnorm_args;
+int t5a_rmsnorm(const t5a_rmsnorm_args* args, t5a_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

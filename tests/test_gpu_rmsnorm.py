@@ -1,0 +1,73 @@
+"""GPU parity of the fused RMS norm / side-token producer against the CPU oracle (through the C ABI)."""
+import pytest
+import torch
+
+from oracle import t5_basic as O
+from oracle.t5_model import tglobal_side_inputs
+
+pytestmark = pytest.mark.gpu
+
+DT = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}
+
+
+@pytest.mark.parametrize("xdt,wdt", [("bf16", "bf16"), ("f32", "f32"), ("f32", "bf16"), ("bf16", "f32"), ("f16", "f16")])
+@pytest.mark.parametrize("shape", [(2, 100, 768), (3, 7, 512), (1, 16384, 768), (5, 4096), (2, 9, 64), (4, 33, 4096)])
+def test_rms_norm_matches_the_oracle(gpu_device, xdt, wdt, shape):
+    from turbot5_amd.ops import rms_norm
+    g = torch.Generator().manual_seed(sum(shape) + len(xdt) * 7 + len(wdt))
+    x = (2.0 * torch.randn(*shape, generator=g)).to(DT[xdt])
+    w = (1.0 + 0.2 * torch.randn(shape[-1], generator=g)).to(DT[wdt])
+    want = O.rms_norm(x, w, 1e-6)
+    got = rms_norm(x.to(gpu_device), w.to(gpu_device), 1e-6)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    diff = (got.float().cpu() - want.float()).abs()
+    if want.dtype == torch.float32:
+        assert (diff <= 2e-6 + 1e-5 * want.float().abs()).all()
+    else:
+        # two roundings (scaled value, then product): a last-bit difference of the fp32 scale can move the
+        # result by up to two units in the last place; it almost never does
+        ulp = 2.0 ** -7 if want.dtype == torch.bfloat16 else 2.0 ** -10
+        assert (diff <= 2 * ulp * want.float().abs() + 1e-6).all()
+        assert (diff == 0).float().mean().item() > 0.98
+
+
+def test_rms_norm_strided_rows_and_closed_form(gpu_device):
+    from turbot5_amd.ops import rms_norm
+    big = torch.randn(4, 50, 1024, generator=torch.Generator().manual_seed(3))
+    x = big[:, :, 256:768]                                           # row stride 1024, 512 columns
+    w = torch.ones(512)
+    got = rms_norm(x.to(gpu_device)[:, :, :], w.to(gpu_device)).cpu()
+    assert torch.allclose(got.pow(2).mean(-1), torch.ones(4, 50), atol=1e-4)   # unit RMS by definition
+    assert torch.allclose(got, O.rms_norm(x, w), atol=1e-5, rtol=1e-5)
+    const = torch.full((3, 64), 5.0)                                 # constant row -> weight itself
+    w2 = torch.linspace(-1, 1, 64)
+    assert torch.allclose(rms_norm(const.to(gpu_device), w2.to(gpu_device), 0.0).cpu(), w2.expand(3, 64), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("L,gbs", [(512, 16), (100, 16), (37, 8), (16, 16), (15, 16), (2048, 1), (130, 64)])
+def test_side_token_producer_matches_the_oracle(gpu_device, dtype, L, gbs):
+    """Block sums + norm in one kernel, against the one-hot einsum + norm of the oracle; L % gbs != 0
+    exercises the orphan tokens that join the last full block."""
+    from turbot5_amd.ops import rms_norm
+    B, d = 3, 256
+    g = torch.Generator().manual_seed(L * 31 + gbs)
+    hidden = torch.randn(B, L, d, generator=g).to(DT[dtype])
+    w = (1.0 + 0.1 * torch.randn(d, generator=g)).to(DT[dtype])
+    want = tglobal_side_inputs(hidden, gbs, w, 1e-6)
+    got = rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=gbs)
+    assert got.shape == want.shape == (B, L // gbs, d)
+    if want.numel():
+        tol = 1e-5 if dtype == "f32" else 2e-2                        # bf16: the einsum's accumulation order is free
+        assert (got.float().cpu() - want.float()).abs().max().item() <= tol * max(1.0, want.float().abs().max().item())
+
+
+def test_layer_norm_module_uses_the_kernel(gpu_device):
+    from turbot5_amd.attentions import T5LayerNorm
+    torch.manual_seed(0)
+    m = T5LayerNorm(768).to(gpu_device).to(torch.bfloat16)
+    x = torch.randn(2, 300, 768).to(torch.bfloat16)
+    want = O.rms_norm(x, m.weight.detach().cpu(), m.eps)
+    got = m(x.to(gpu_device))
+    assert got.dtype == torch.bfloat16
+    assert (got.float().cpu() - want.float()).abs().max().item() <= 2.0 ** -6

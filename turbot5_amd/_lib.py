@@ -17,7 +17,7 @@ PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
-    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk",
+    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_rmsnorm",
 )
 
 
@@ -68,6 +68,13 @@ class T5ASplitKArgs(C.Structure):
                 ("D", C.c_int32), ("num_splits", C.c_int32), ("sm_scale", C.c_float)]
 
 
+class T5ARmsNormArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("weight", C.c_void_p), ("y", C.c_void_p),
+                ("x_strides", C.c_int64 * 2),
+                ("batches", C.c_int64), ("rows_per_batch", C.c_int32), ("dim", C.c_int32), ("group", C.c_int32),
+                ("x_dtype", C.c_int32), ("weight_dtype", C.c_int32), ("eps", C.c_float)]
+
+
 _lib = None
 _lock = threading.Lock()
 
@@ -102,6 +109,8 @@ def load() -> C.CDLL:
             fn.restype = C.c_int
         lib.t5a_splitk_workspace_bytes.argtypes = [C.c_int32] * 5
         lib.t5a_splitk_workspace_bytes.restype = C.c_int64
+        lib.t5a_rmsnorm.argtypes = [C.POINTER(T5ARmsNormArgs), C.c_void_p]
+        lib.t5a_rmsnorm.restype = C.c_int
         lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7
         lib.t5a_sparse_workspace_bytes.restype = C.c_int64
         _lib = lib

@@ -41,7 +41,20 @@ class T5LayerNorm(nn.Module):
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(dim))
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, group: int = 1) -> torch.Tensor:
+        """On a ROCm device: the fused HIP kernel (the reference switches to its Triton kernel there,
+        modules.py:61-66).  Host tensors take the reference's eager formula (modules.py:51-59).
+        ``group`` > 1 norms the sums of ``group`` consecutive rows of each sequence (side tokens)."""
+        if x.is_cuda:
+            from .ops import rms_norm
+            return rms_norm(x, self.weight, self.eps, group)
+        if group > 1:
+            B, L, d = x.shape
+            n = L // group
+            agg = x[:, :n * group].reshape(B, n, group, d).sum(dim=2)
+            if L > n * group and n > 0:
+                agg = torch.cat([agg[:, :-1], agg[:, -1:] + x[:, n * group:].sum(dim=1, keepdim=True)], dim=1)
+            x = agg
         variance = x.to(torch.float32).pow(2).mean(-1, keepdim=True)
         x = x * torch.rsqrt(variance + self.eps)
         if self.weight.dtype in (torch.float16, torch.bfloat16):
@@ -289,11 +302,7 @@ class T5TransientGlobalAttention(_SparseBase):
         n_side = L // gbs
         if n_side == 0:
             return hidden_states.new_zeros(B, 0, d)
-        full = n_side * gbs
-        agg = hidden_states[:, :full].reshape(B, n_side, gbs, d).sum(dim=2)
-        if L > full:
-            agg = torch.cat([agg[:, :-1], agg[:, -1:] + hidden_states[:, full:].sum(dim=1, keepdim=True)], dim=1)
-        return self.global_input_layer_norm(agg)
+        return self.global_input_layer_norm(hidden_states, group=gbs)   # block sums and norm in one kernel
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):

@@ -401,4 +401,30 @@ int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
     return finish(launch_splitk(p, a->dtype, a->D, (hipStream_t)stream), "t5a_fwd_splitk");
 }
 
+int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    for (int dt : {a->x_dtype, a->weight_dtype})
+        if (dt != T5A_BF16 && dt != T5A_F16 && dt != T5A_F32) return fail(T5A_ERR_DTYPE, "unsupported dtype %d", dt);
+    if (a->batches < 0 || a->rows_per_batch < 0 || a->dim <= 0 || a->group < 1)
+        return fail(T5A_ERR_SHAPE, "bad sizes batches=%lld rows=%d dim=%d group=%d", (long long)a->batches, a->rows_per_batch, a->dim, a->group);
+    if (a->dim % 8 != 0) return fail(T5A_ERR_SHAPE, "dim=%d must be a multiple of 8", a->dim);
+    const int out_per_batch = a->rows_per_batch / a->group;
+    if (a->batches == 0 || out_per_batch == 0) return T5A_OK;
+    if (a->x == nullptr || a->weight == nullptr || a->y == nullptr) return fail(T5A_ERR_NULL, "x, weight or y is NULL");
+    if (!aligned16(a->x) || (reinterpret_cast<uintptr_t>(a->y) & 31u) != 0) return fail(T5A_ERR_STRIDE, "x must be 16-byte and y 32-byte aligned");
+    const int xunit = a->x_dtype == T5A_F32 ? 4 : 8;
+    if (a->x_strides[0] % xunit != 0 || a->x_strides[1] % xunit != 0)
+        return fail(T5A_ERR_STRIDE, "x strides must be multiples of %d elements", xunit);
+    RmsParams p;
+    memset(&p, 0, sizeof(p));
+    p.x = a->x; p.weight = a->weight; p.y = a->y;
+    p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;
+    p.out_per_batch = out_per_batch;
+    p.out_rows = a->batches * out_per_batch;
+    p.rows_per_batch = a->rows_per_batch; p.group = a->group; p.dim = a->dim;
+    p.eps = a->eps;
+    if ((p.out_rows + 3) / 4 > 0x7fffffffLL) return fail(T5A_ERR_SHAPE, "too many rows (%lld)", (long long)p.out_rows);
+    return finish(launch_rmsnorm(p, a->x_dtype, a->weight_dtype, (hipStream_t)stream), "t5a_rmsnorm");
+}
+
 }  // extern "C"

@@ -71,4 +71,14 @@ hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t st
 // only the merge over splits (part_o, part_l, part_m -> o)
 hipError_t launch_splitk_merge(const SplitKParams& p, int dtype, int D, hipStream_t stream);
 
+struct RmsParams {
+    const void* x; const void* weight; void* y;
+    int64_t x_batch_stride, x_row_stride, y_row_stride;   // elements
+    int64_t out_rows;        // batches * out_per_batch
+    int out_per_batch;       // rows_per_batch / group (group == 1: rows_per_batch)
+    int rows_per_batch, group, dim;
+    float eps;
+};
+hipError_t launch_rmsnorm(const RmsParams& p, int x_dtype, int w_dtype, hipStream_t stream);
+
 }  // namespace t5a

@@ -212,6 +212,46 @@ def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, b
                    NUM_BUCKETS, MAX_DISTANCE)
 
 
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1) -> torch.Tensor:
+    """T5 RMS norm over the last dimension (src/turbot5/model/modules.py:51-59).
+
+    ``group`` > 1: x is (B, L, d) and row r of the (B, L // group, d) result is the norm of the sum of
+    rows [r*group, (r+1)*group) of its sequence, trailing rows joining the last group: the side-token
+    producer of transient-global attention (src/turbot5/model/utils.py:249-258, :206-212).
+    The result has the weight's dtype when that is 16 bit, else fp32, as torch promotes the reference code."""
+    if not (x.is_cuda and weight.is_cuda):
+        raise RuntimeError("x and weight must be on a ROCm device: this path has no CPU implementation")
+    d = x.shape[-1]
+    if weight.shape != (d,):
+        raise ValueError(f"weight must have shape ({d},), got {tuple(weight.shape)}")
+    out_dtype = weight.dtype if weight.dtype in (torch.float16, torch.bfloat16) else torch.float32
+    w = weight.detach().contiguous()
+    x_ = x.detach()
+    if group == 1:
+        x2 = x_.reshape(-1, d)
+        if x2.stride(-1) != 1 or x2.stride(0) % 8 != 0 or x2.data_ptr() % 16 != 0:
+            x2 = x2.contiguous()
+        batches, rows, strides = 1, x2.shape[0], (0, x2.stride(0))
+        out_shape = x.shape
+    else:
+        if x_.dim() != 3:
+            raise ValueError("grouped rms_norm needs x of shape (B, L, d)")
+        x2 = x_
+        if x2.stride(-1) != 1 or x2.stride(0) % 8 != 0 or x2.stride(1) % 8 != 0 or x2.data_ptr() % 16 != 0:
+            x2 = x2.contiguous()
+        batches, rows, strides = x2.shape[0], x2.shape[1], (x2.stride(0), x2.stride(1))
+        out_shape = (x2.shape[0], rows // group, d)
+    y = torch.empty(out_shape, dtype=out_dtype, device=x.device)
+    a = L.T5ARmsNormArgs()
+    a.x, a.weight, a.y = x2.data_ptr(), w.data_ptr(), y.data_ptr()
+    a.x_strides = (C.c_int64 * 2)(*strides)
+    a.batches, a.rows_per_batch, a.dim, a.group = batches, rows, d, int(group)
+    a.x_dtype, a.weight_dtype, a.eps = _dtype_code(x2), _dtype_code(w), float(eps)
+    with torch.cuda.device(x.device):
+        L.check(L.load().t5a_rmsnorm(C.byref(a), _stream(x)))
+    return y
+
+
 def default_num_splits(B: int, H: int, N: int, device=None) -> int:
     """Enough splits to give every compute unit a few workgroups, at least 256 keys per split."""
     cus = 256
