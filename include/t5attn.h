@@ -106,12 +106,18 @@ int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
  * q,o: (total_q,H,D); k,v: (total_k,H,D); strides = {row, head}.
  * cu_seqlens_q/k: DEVICE int32 arrays of B+1 ascending offsets.  Positions are
  * in-sequence; per sequence the semantics equal t5a_fwd_dense.
+ * seq_lens_q/k (optional): DEVICE int32 arrays of B lengths.  When given, sequence b is
+ * rows [cu[b], cu[b] + lens[b]) and the rows up to cu[b+1] are padding that is neither read
+ * nor written: a right-padded (B,L,H,D) batch runs in place with cu = {0, L, 2L, ...} and
+ * lens = mask.sum(-1), without the gathers and the scatter of the reference's unpad / pad
+ * (src/turbot5/model/padding.py:113-150, :30-44).
  * lse (optional) is (total_q,H) contiguous fp32.
  */
 typedef struct t5a_varlen_args {
     const void* q; const void* k; const void* v; void* o; float* lse;
     int64_t q_strides[2]; int64_t k_strides[2]; int64_t v_strides[2]; int64_t o_strides[2];
     const int32_t* cu_seqlens_q; const int32_t* cu_seqlens_k;
+    const int32_t* seq_lens_q; const int32_t* seq_lens_k;
     int32_t dtype; int32_t B; int32_t H; int32_t D;
     int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
     int32_t causal; float sm_scale;

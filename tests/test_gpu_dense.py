@@ -138,6 +138,35 @@ def test_varlen(gpu_device, causal, dtype):
     assert lse.shape == (tot, H) and torch.isfinite(lse).all()
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_padded_batch_in_place_with_seq_lens(gpu_device, causal):
+    """Right-padded (B, L, H, D) batch viewed as (B*L, H, D): cu = b*L, lengths given separately.  Valid rows
+    equal the packed oracle on the unpadded sequences; padding rows are never read (poisoned with NaN) and
+    come back as zeros, like the reference's pad_input (padding.py:30-44)."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    B, L, H, D = 5, 200, 3, 64
+    lens = [200, 1, 0, 129, 77]
+    q, k, v = (rnd(B, L, H, D, seed=40 + i, dtype=torch.bfloat16) for i in range(3))
+    table = rnd(32, H, seed=43, scale=1.0)
+    for b, n in enumerate(lens):
+        for t in (q, k, v):
+            t[b, n:] = float("nan")
+    cu_pad = torch.arange(0, (B + 1) * L, L, dtype=torch.int32)
+    out, lse = flash_attention_with_fusing_bias_varlen(
+        q.view(B * L, H, D).to(gpu_device), k.view(B * L, H, D).to(gpu_device), v.view(B * L, H, D).to(gpu_device),
+        table.to(gpu_device), cu_pad.to(gpu_device), cu_pad.to(gpu_device), L, L, causal=causal, sm_scale=1.0,
+        return_lse=True, seq_lens_q=torch.tensor(lens, dtype=torch.int32, device=gpu_device),
+        seq_lens_k=torch.tensor(lens, dtype=torch.int32, device=gpu_device))
+    out = out.float().cpu().view(B, L, H, D)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    packed = [torch.cat([t[b, :n] for b, n in enumerate(lens)]) for t in (q, k, v)]
+    want = O.varlen_attention(*packed, table, cu, cu, causal, 1.0)
+    for b, n in enumerate(lens):
+        assert (out[b, :n] - want[cu[b]:cu[b + 1]]).abs().max().item() <= 2e-2 if n else True
+        assert (out[b, n:] == 0).all()
+    assert torch.isfinite(lse).all()
+
+
 def test_varlen_cross_lengths(gpu_device):
     """different q and k lengths per sequence (decoder step over a padded cache)."""
     from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen

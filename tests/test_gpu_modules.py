@@ -68,7 +68,7 @@ def test_attention_module_output_tuple(gpu_device):
 
 
 def test_flash_encoder_with_padding(gpu_device):
-    """A padded batch takes the packed (cu_seqlens) kernel; padded rows come back as zeros."""
+    """A right-padded batch runs in place through the packed kernel with per-sequence lengths."""
     cfg, m, sd = make(dict(SMALL, attention_type="flash"))
     ids = torch.randint(0, 200, (3, 150), generator=torch.Generator().manual_seed(2))
     mask = torch.ones(3, 150)
@@ -80,6 +80,27 @@ def test_flash_encoder_with_padding(gpu_device):
         got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
     valid = mask.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+
+
+def test_flash_encoder_with_left_padding_and_holes(gpu_device):
+    """A mask that is not a run of ones followed by zeros cannot run in place: it takes the gather /
+    packed kernel / scatter route (the reference's only route, attentions.py:492-511).  As in the
+    reference, positions are counted over the VALID tokens of a sequence (padding.py:113-150 packs them
+    before the kernel numbers them, varlen_fused_bias_attn.py:254, :303), so each sequence equals the
+    oracle run on its valid tokens alone."""
+    cfg, m, sd = make(dict(SMALL, attention_type="flash"))
+    ids = torch.randint(0, 200, (3, 140), generator=torch.Generator().manual_seed(5))
+    mask = torch.ones(3, 140)
+    mask[0, :30] = 0                 # left padding
+    mask[1, 50:60] = 0               # a hole
+    mask[2, 100:] = 0                # right padding in the same batch
+    m = m.to(gpu_device)
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
+    for b in range(3):
+        valid = mask[b].bool()
+        want = OM.encoder_forward(sd, cfg, ids[b][valid][None])[0]
+        assert (got[b][valid] - want).abs().max().item() <= 2e-3
 
 
 def test_bf16_attention_inside_fp32_model(gpu_device):

@@ -41,6 +41,7 @@ class T5AVarlenArgs(C.Structure):
                 ("q_strides", C.c_int64 * 2), ("k_strides", C.c_int64 * 2), ("v_strides", C.c_int64 * 2),
                 ("o_strides", C.c_int64 * 2),
                 ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
+                ("seq_lens_q", C.c_void_p), ("seq_lens_k", C.c_void_p),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32),
                 ("max_seqlen_k", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),

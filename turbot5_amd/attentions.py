@@ -76,8 +76,16 @@ def _mask_info(mask: torch.Tensor):
         return hit
     if mask.dim() != 2:
         raise ValueError(f"attention mask must be (batch, key_length) of 0/1, got shape {tuple(mask.shape)}")
-    all_ones = bool((mask != 0).all())
-    unpad = None if all_ones else _get_unpad_data((mask != 0).to(torch.int32))
+    valid = mask != 0
+    lens = valid.sum(-1, dtype=torch.int32)
+    steps = torch.arange(mask.shape[1], device=mask.device)
+    # one transfer for both questions: all ones?  right-padded (every row a run of ones, then zeros)?
+    all_ones, right_padded = (bool(x) for x in torch.stack(
+        [valid.all(), (valid == (steps[None, :] < lens[:, None])).all()]).tolist())
+    unpad = None
+    if not all_ones:
+        # right-padded batches run in place with per-sequence lengths; anything else is packed first
+        unpad = ("lens", lens) if right_padded else ("packed", _get_unpad_data(valid.to(torch.int32)))
     _MASK_INFO[key] = (all_ones, unpad)
     while len(_MASK_INFO) > 16:
         _MASK_INFO.popitem(last=False)
@@ -192,7 +200,24 @@ class T5FlashAttention(_T5AttentionBase):
             q_blhd = query_states.transpose(1, 2)
             k_blhd = key_states.transpose(1, 2)
             v_blhd = value_states.transpose(1, 2)
-            if key_value_states is None and seq_length == key_length:
+            kind, unpad = unpad
+            dev = hidden_states.device
+            if kind == "lens":
+                # right-padded batch: the kernel walks the padded (B*L, H, D) layout with per-sequence
+                # lengths; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
+                def rows(t, n):
+                    t = t if t.is_contiguous() else t.contiguous()
+                    return t.view(batch_size * n, self.n_heads, -1)
+                cu_k = torch.arange(0, (batch_size + 1) * key_length, key_length, dtype=torch.int32, device=dev)
+                self_attn = key_value_states is None and seq_length == key_length
+                cu_q = cu_k if self_attn else torch.arange(0, (batch_size + 1) * seq_length, seq_length,
+                                                           dtype=torch.int32, device=dev)
+                out_p = ops.flash_attention_with_fusing_bias_varlen(
+                    rows(q_blhd, seq_length), rows(k_blhd, key_length), rows(v_blhd, key_length), table, cu_q, cu_k,
+                    seq_length, key_length, causal=self.causal, sm_scale=1.0, NUM_BUCKETS=nb, MAX_DISTANCE=md,
+                    seq_lens_q=unpad if self_attn else None, seq_lens_k=unpad)
+                attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
+            elif key_value_states is None and seq_length == key_length:
                 q_p, k_p, v_p, indices_q, (cu_q, cu_k), (max_q, max_k) = _upad_input(
                     q_blhd, k_blhd, v_blhd, mask, seq_length, self.n_heads, unpad_data=unpad)
             else:
@@ -204,13 +229,14 @@ class T5FlashAttention(_T5AttentionBase):
                 cu_q = torch.arange(0, (batch_size + 1) * seq_length, seq_length, dtype=torch.int32,
                                     device=hidden_states.device)
                 indices_q, max_q = None, seq_length
-            out_p = ops.flash_attention_with_fusing_bias_varlen(
-                q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
-                NUM_BUCKETS=nb, MAX_DISTANCE=md)
-            if indices_q is not None:
-                attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
-            else:
-                attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
+            if kind != "lens":
+                out_p = ops.flash_attention_with_fusing_bias_varlen(
+                    q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
+                    NUM_BUCKETS=nb, MAX_DISTANCE=md)
+                if indices_q is not None:
+                    attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
+                else:
+                    attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
 
         attn_output = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
         present_key_value_state = (key_states, value_states) if (self.is_decoder and use_cache) else None

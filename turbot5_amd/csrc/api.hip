@@ -232,6 +232,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     p.o_sr = a->o_strides[0]; p.o_sh = a->o_strides[1];
     p.lse_sr = a->H; p.lse_sh = 1;
     p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+    p.len_q = a->seq_lens_q; p.len_k = a->seq_lens_k;
     p.B = a->B; p.H = a->H; p.M = a->max_seqlen_q; p.N = a->max_seqlen_k;
     // sum_b ceil(len_b / 128) <= total_q / 128 + B: launch that many, the surplus exits
     const int64_t items = ((int64_t)a->total_q / 128 + a->B) * a->H;

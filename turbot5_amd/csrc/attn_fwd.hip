@@ -283,7 +283,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         b = -1;
         for (int bb = 0; bb < p.B; ++bb) {
             qs = p.cu_q[bb];
-            const int len = p.cu_q[bb + 1] - qs;
+            const int len = p.len_q != nullptr ? p.len_q[bb] : p.cu_q[bb + 1] - qs;
             nt_b = (len + BM - 1) / BM;
             const int cnt = nt_b * p.H;
             if (w < acc + cnt) { b = bb; Mseq = len; w -= acc; break; }
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         qt = w - h * nt_b;
         if (CAUSAL) qt = nt_b - 1 - qt;
         const int ks = p.cu_k[b];
-        Nseq = p.cu_k[b + 1] - ks;
+        Nseq = p.len_k != nullptr ? p.len_k[b] : p.cu_k[b + 1] - ks;
         q_off = (int64_t)qs * p.q_sr + (int64_t)h * p.q_sh;
         o_off = (int64_t)qs * p.o_sr + (int64_t)h * p.o_sh;
         k_off = (int64_t)ks * p.k_sr + (int64_t)h * p.k_sh;

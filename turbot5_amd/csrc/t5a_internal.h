@@ -35,6 +35,7 @@ struct FwdParams {
     int64_t sv_sb, sv_sh, sv_sr;
     int64_t lse_sb, lse_sh, lse_sr;
     const int32_t* cu_q; const int32_t* cu_k;   // non-null: packed variable-length batch
+    const int32_t* len_q; const int32_t* len_k; // optional lengths (rows between cu[b]+len[b] and cu[b+1] are padding)
     int B, H, M, N;
     int tiles_per_seq;   // q tiles per (batch, head) when not packed
     int total_items;     // number of (q tile, head, batch) work items (upper bound when packed)

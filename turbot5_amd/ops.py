@@ -111,11 +111,16 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
 
 def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                             causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                            return_lse: bool = False):
+                                            return_lse: bool = False, seq_lens_q=None, seq_lens_k=None):
     """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
 
     Positions restart at 0 in every sequence.  No host synchronisation: the
     work list is derived on the device from ``cu_seqlens``.
+
+    ``seq_lens_q`` / ``seq_lens_k`` (optional int32 device tensors of B lengths): sequence b is rows
+    [cu[b], cu[b] + lens[b]); the rows up to cu[b+1] are padding, never read and left ZERO in the
+    output.  A right-padded (B, L, H, D) batch runs in place this way, viewed as (B*L, H, D) with
+    cu = arange(B+1) * L and lens = mask.sum(-1): no gathers, no scatter.
     """
     _check_inputs(q, k, v)
     total_q, H, D = q.shape
@@ -130,14 +135,26 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     cq = cu_seqlens_q.to(device=q.device, dtype=torch.int32).contiguous()
     ck = cq if cu_seqlens_k is cu_seqlens_q else cu_seqlens_k.to(device=q.device, dtype=torch.int32).contiguous()
     q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
-    o = torch.empty_like(q_)
-    lse = torch.empty((total_q, H), device=q.device, dtype=torch.float32) if return_lse else None
+    lens = []
+    for t in (seq_lens_q, seq_lens_k):
+        if t is not None:
+            if t.numel() != B:
+                raise ValueError(f"seq_lens must hold {B} lengths, got {t.numel()}")
+            t = t.to(device=q.device, dtype=torch.int32).contiguous()
+        lens.append(t)
+    # padding rows are not written by the kernel: they read as zeros, like the reference's pad_input
+    o = torch.empty_like(q_) if lens[0] is None else torch.zeros_like(q_)
+    lse = None
+    if return_lse:
+        lse = (torch.empty if lens[0] is None else torch.zeros)((total_q, H), device=q.device, dtype=torch.float32)
     a = L.T5AVarlenArgs()
     a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
     a.lse = lse.data_ptr() if lse is not None else None
     for name, t in (("q_strides", q_), ("k_strides", k_), ("v_strides", v_), ("o_strides", o)):
         setattr(a, name, (C.c_int64 * 2)(t.stride(0), t.stride(1)))
     a.cu_seqlens_q, a.cu_seqlens_k = cq.data_ptr(), ck.data_ptr()
+    a.seq_lens_q = lens[0].data_ptr() if lens[0] is not None else None
+    a.seq_lens_k = lens[1].data_ptr() if lens[1] is not None else None
     a.dtype, a.B, a.H, a.D = _dtype_code(q), B, H, D
     a.total_q, a.total_k = total_q, total_k
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
