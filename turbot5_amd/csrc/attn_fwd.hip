@@ -110,17 +110,6 @@ constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 #ifndef OCC
 #define OCC 2
 #endif
-#ifndef T5A_PRIO
-#define T5A_PRIO 0
-#endif
-#ifndef T5A_SGB
-#define T5A_SGB 0
-#endif
-#ifdef ABL_NOEXP
-#define ABL_EXP(x) (x)
-#else
-#define ABL_EXP(x) __builtin_amdgcn_exp2f(x)
-#endif
 
 __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
     int out = 0, d;
@@ -684,9 +673,6 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
             c.skip = t >= d_ts;
             const bool left_sat = t < d_tl, right_sat = t >= d_tr;
             c.use_lut = has_lut && !(left_sat || right_sat);
-#ifdef ABL_NOLUTTILE
-            c.use_lut = false;
-#endif
             c.need_mask = t >= d_tm;
             c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
             return c;
@@ -748,11 +734,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
                 const int row = 32 * nt + lr;
 #pragma unroll
                 for (int s = 0; s < KS; ++s)
-#ifdef ABL_NOLDS
-                    ka[nt][s] = qf[(s + nt) % KS];
-#else
                     ka[nt][s] = *reinterpret_cast<const v8*>(ks + row * D + (((2 * s + hh) ^ G::kswz(row)) * 8));
-#endif
             }
         }
     };
@@ -875,7 +857,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
                 for (int u = 0; u < 2; ++u) {
                     f32x8 pv;
 #pragma unroll
-                    for (int x = 0; x < 8; ++x) pv[x] = ABL_EXP(st[nt][8 * u + x]);
+                    for (int x = 0; x < 8; ++x) pv[x] = __builtin_amdgcn_exp2f(st[nt][8 * u + x]);
                     const v8 pb = __builtin_convertvector(pv, v8);
                     if (u == 0) l_run = E::sum8(pb, l_run); else l_alt = E::sum8(pb, l_alt);
 #pragma unroll
@@ -886,11 +868,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
                         const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#ifdef ABL_NOLDS
-                        ot[dt] = E::mfma(qf[(dt + u) % KS], pb, ot[dt]);
-#else
                         ot[dt] = E::mfma(__builtin_bit_cast(v8, both), pb, ot[dt]);
-#endif
                     }
                 }
         } else if constexpr (F32) {
@@ -913,7 +891,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
                 for (int u = 0; u < 2; ++u) {
                     f32x8 pv;
 #pragma unroll
-                    for (int x = 0; x < 8; ++x) pv[x] = ABL_EXP(st[nt][8 * u + x]);
+                    for (int x = 0; x < 8; ++x) pv[x] = __builtin_amdgcn_exp2f(st[nt][8 * u + x]);
                     const v8 pb = __builtin_convertvector(pv, v8);
                     if (u == 0) l_run = E::sum8(pb, l_run); else l_alt = E::sum8(pb, l_alt);
 #pragma unroll
@@ -965,10 +943,8 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         const int kbuf_next = DMA ? (t + 1) % NSK : (t + 1) & 1;
         const int vbuf = DMA ? t % NSV : t & 1;
         if constexpr (DMA) {
-#ifndef ABL_NOLOAD
             dma_tile(t + 4, false);
             dma_tile(t + 3, true);
-#endif
         } else {
             if (t + 2 < ntiles) load_tile_k(t + 2);
             if (t + 1 < ntiles) load_tile_v(t + 1);
@@ -983,12 +959,8 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         if (!tc.skip) compute_pv(vbuf, st);
         tc = nx;
         if constexpr (DMA) {
-#ifndef ABL_NOLOAD
             __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8): everything but the last two steps' requests
-#endif
-#ifndef ABL_NOBAR
             barrier_lds_only();
-#endif
         } else {
             if (t + 2 < ntiles) store_tile_k(t & 1);
             if (t + 1 < ntiles) store_tile_v((t + 1) & 1);
