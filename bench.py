@@ -149,6 +149,14 @@ def extra_workloads(torch, dev, steps, full):
         mem = torch.randn(64, 8192, 768, generator=torch.Generator().manual_seed(6)).to(dev)
         steps_dec = 64
         with torch.no_grad():
+            # the baseline's end-to-end case: 100k-token encoder input, 128-token decoder, fp32 activations, bf16 attention
+            ids = torch.randint(0, 32128, (1, 100000), generator=torch.Generator().manual_seed(8)).to(dev)
+            dec_ids = torch.randint(0, 32128, (1, 128), generator=torch.Generator().manual_seed(9)).to(dev)
+            f = lambda: model(ids, dec_ids)  # noqa: E731
+            _, ms = time_kernel(torch, f, 2, 1)
+            out["t5_base_encdec_100k_enc_128_dec_fp32_act_bf16_attn"] = {
+                "ms": round(ms, 1), "encoder_tokens_per_s": round(1e5 / (ms * 1e-3), 1)}
+            del ids, dec_ids
             model.greedy_decode(encoder_outputs=mem, max_new_tokens=4)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
