@@ -99,9 +99,10 @@ template <> struct Elem<float> {
 };
 
 constexpr int BM = 128;      // query rows per workgroup
-constexpr int BN = 64;       // keys per tile
+// keys per tile: 64, or 32 at head_dim 128 (16-bit types), where the halved score registers and K/V
+// tiles keep two workgroups per compute unit
+template <typename T, int D> constexpr int tile_keys() { return sizeof(T) == 2 && D == 128 ? 32 : 64; }
 constexpr int NTHREADS = 256;
-constexpr int NT = BN / 32;  // 32-key blocks per tile
 // The distance LUT extends this far past the saturation distance on both sides.  A tile that takes
 // the LUT path has at least one unsaturated (row, key) pair, and a wavefront tile spans 32 rows x
 // 64 keys, so none of its distances lies more than 94 past saturation: lookups need no clamping.
@@ -181,6 +182,12 @@ __device__ __forceinline__ void lds_dma_16x2(unsigned lo, unsigned hi, unsigned 
                  :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory");
 }
 
+// s_waitcnt vmcnt(N) alone (six-bit count: bits 3:0 and 15:14), the other counters left open
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
 // barrier that orders LDS traffic only (lgkmcnt), leaving LDS-DMA requests in flight
 __device__ __forceinline__ void barrier_lds_only() {
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
@@ -194,6 +201,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 template <typename T, int D>
 struct Geometry {
     static constexpr bool F32 = sizeof(T) == 4;
+    static constexpr int BN = tile_keys<T, D>();
+    static constexpr int NT = BN / 32;                  // 32-key blocks per tile
     static constexpr int EPC = 16 / sizeof(T);         // elements per 16-byte chunk
     static constexpr int KS = F32 ? D / 2 : D / 16;    // k-steps of the S^T product
     static constexpr int DT = (D + 31) / 32;           // 32-row blocks of O^T
@@ -208,9 +217,13 @@ struct Geometry {
     static constexpr int KSTR = F32 ? D + 1 : D;       // fp32 K rows padded by one float (bank spread)
     static constexpr int K_TILE = BN * KSTR;
     static constexpr int V_TILE = VROWS * BN;          // 16-bit: V^T (dim x key); fp32: V (key x VROWS)
-    // 16-bit types with 128-byte rows are staged by LDS-DMA (buffer loads that write LDS directly):
+    // 16-bit types with 128- or 256-byte rows are staged by LDS-DMA (buffer loads that write LDS directly):
     // no staging registers, no vector ALU work, V stays row-major and is transposed on the LDS read.
-    static constexpr bool DMA = !F32 && D == 64;
+    static constexpr bool DMA = !F32 && (D == 64 || D == 128);
+    // one request of a wavefront moves 1 KB: RPS whole rows of LPR lanes each; a tile is SPW such slabs per wavefront
+    static constexpr int LPR = D / 8 > 0 ? D / 8 : 1;
+    static constexpr int RPS = 64 / LPR;
+    static constexpr int SPW = BN * D / 2048 > 0 ? BN * D / 2048 : 1;
     static constexpr int NSK = DMA ? 4 : 2;             // LDS stages of K
     static constexpr int NSV = DMA ? 4 : 2;             // LDS stages of V
     static constexpr size_t kTileBytes = (size_t)(NSK * K_TILE + NSV * V_TILE) * sizeof(T);
@@ -222,7 +235,8 @@ struct Geometry {
     static __device__ __forceinline__ int vswz(int d) { return ((d >> 1) & 7) ^ ((d >> 4) & 7); }
     // row-major V (LDS-DMA path): the transposing read of a half wavefront touches 4 consecutive
     // keys x 64 bytes; flipping the 64-byte halves of keys 2,3 (mod 4) spreads them over all banks
-    static __device__ __forceinline__ int vrow_swz(int key) { return ((key >> 1) & 1) << 2; }
+    // (rows of 256 bytes span all banks: there the four keys of a read go to four different quarters)
+    static __device__ __forceinline__ int vrow_swz(int key) { return D == 128 ? (key & 3) << 2 : ((key >> 1) & 1) << 2; }
 };
 
 // floats per shifted copy of the distance LUT (host and device agree through this)
@@ -232,7 +246,7 @@ __host__ __device__ inline int lut_quads(int sat, bool causal) {
 }
 
 template <typename T, int D, int MODE, bool CAUSAL>
-__global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
     using v8 = typename E::v8;
@@ -242,6 +256,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
     constexpr int K_CHUNKS = G::K_CHUNKS, K_PER_T = G::K_PER_T, V_UNITS = G::V_UNITS, V_PER_T = G::V_PER_T;
     constexpr int KSTR = G::KSTR, K_TILE = G::K_TILE, V_TILE = G::V_TILE;
     constexpr int ES = sizeof(T);
+    constexpr int BN = G::BN, NT = G::NT;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr bool DMA = G::DMA;
@@ -404,9 +419,9 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
             if (stage < 0) stage = is_v ? t % NSV : t % NSK;
             const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int slab = wave * 2 + c;              // 1 KB = 8 rows
-                const int r = slab * 8 + (lane >> 3), pc = lane & 7;
+            for (int c = 0; c < G::SPW; ++c) {
+                const int slab = wave * G::SPW + c;         // 1 KB = RPS rows
+                const int r = slab * G::RPS + lane / G::LPR, pc = lane % G::LPR;
                 const int ch = pc ^ (is_v ? G::vrow_swz(r) : G::kswz(r));
                 lds_dma_16(rs, base + slab * 1024, (j0 + r) * sr + ch * 16);
             }
@@ -419,13 +434,16 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
     unsigned long long kcur = 0, vcur = 0;
     int kleft = 0, vleft = 0;
     const int kstep = BN * seg_ksr[0], vstep = BN * seg_vsr[0];
-    int cur_koff[2] = {0, 0}, cur_voff[2] = {0, 0};
+    int cur_koff[G::SPW], cur_voff[G::SPW];
+#pragma unroll
+    for (int c = 0; c < G::SPW; ++c) cur_koff[c] = cur_voff[c] = 0;
     if constexpr (DMA && MODE == kDense) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int r = (wave * 2 + c) * 8 + (lane >> 3), pc = lane & 7;
-            cur_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16 - c * 1024;
-            cur_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16 - c * 1024;
+        for (int c = 0; c < G::SPW; ++c) {
+            const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
+            // requests go out in pairs; the second of a pair carries an instruction offset of 1024
+            cur_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16 - (c & 1) * 1024;
+            cur_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16 - (c & 1) * 1024;
         }
     }
     auto cursor_seek = [&](int tk, int tv) {   // next requests: K tile tk, V tile tv
@@ -436,11 +454,14 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
     };
     auto cursor_dma = [&](int kstage, int vstage) {
         if constexpr (DMA) {
-            const unsigned wbase = lds_base + (unsigned)wave * 2048u;
-            lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
-                         wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES, cur_koff[0], cur_koff[1]);
-            lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
-                         wbase + (unsigned)(vstage * V_TILE) * ES, cur_voff[0], cur_voff[1]);
+            const unsigned wbase = lds_base + (unsigned)wave * (1024u * G::SPW);
+#pragma unroll
+            for (int c = 0; c < G::SPW; c += 2) {
+                lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
+                             wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES + c * 1024u, cur_koff[c], cur_koff[c + 1]);
+                lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
+                             wbase + (unsigned)(vstage * V_TILE) * ES + c * 1024u, cur_voff[c], cur_voff[c + 1]);
+            }
             kcur += (unsigned)kstep; vcur += (unsigned)vstep;
             kleft -= kstep; vleft -= vstep;
         }
@@ -839,14 +860,16 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
     // per-lane part of the transposing V reads (LDS-DMA path): within a group of 16 lanes, lane
     // r = 4j + a supplies the address of V[key j][4a .. 4a+3] and receives, for head dim (lane % 16),
     // the four keys j = 0..3 -- one 16 x 4 fragment of V^T per read, two reads per MFMA operand.
-    int vtr_off[2] = {0, 0};   // element offsets for dt = 0, 1 (before the per-block constants)
+    int vtr_off[DT];   // element offsets per 32-dim block (before the per-block constants)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vtr_off[dt] = 0;
     if constexpr (DMA) {
         const int g = lane >> 4, r = lane & 15, jj = r >> 2, aa = r & 3;
         const int row = 4 * (g >> 1) + jj;                      // + 32 nt + 16 u (+ 8 for the second read)
         const int x = 2 * (g & 1) + (aa >> 1);
-        const int fb = G::vrow_swz(row) >> 2;                   // 0 or 1: swaps the 64-byte halves
+        const int fb = G::vrow_swz(row) >> 2;                   // which 64-byte part of the row holds block 0
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt) vtr_off[dt] = row * D + ((4 * (dt ^ fb) + x) * 8) + (aa & 1) * 4;
+        for (int dt = 0; dt < DT; ++dt) vtr_off[dt] = row * D + ((4 * (dt ^ fb) + x) * 8) + (aa & 1) * 4;
     }
     auto compute_pv = [&](int buf, f32x16 (&st)[NT]) {
         const T* vs = Vs + buf * V_TILE;
@@ -919,8 +942,9 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
     // ahead and V tiles one step ahead, each in two LDS buffers, with one barrier per step.
     //
     // LDS-DMA path: K(t+4) and V(t+3) are requested in step t into four-stage rings; every step
-    // issues exactly four loads per wavefront (tiles past the end fetch zeros), so "at most eight
-    // loads outstanding" before the barrier means the tiles of the next step have landed.
+    // issues the same number of loads per wavefront (2 * SPW; tiles past the end fetch zeros), so
+    // "at most two steps' worth outstanding" before the barrier means the tiles of the next step
+    // have landed.
     f32x16 sta[NT], stb[NT];
     TileClass tc = classify(0);
     if constexpr (DMA) {
@@ -959,7 +983,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         if (!tc.skip) compute_pv(vbuf, st);
         tc = nx;
         if constexpr (DMA) {
-            __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8): everything but the last two steps' requests
+            wait_vmcnt<4 * G::SPW>();   // everything but the last two steps' requests
             barrier_lds_only();
         } else {
             if (t + 2 < ntiles) store_tile_k(t & 1);
@@ -985,7 +1009,7 @@ __global__ __launch_bounds__(NTHREADS, D >= 128 ? 1 : OCC) void fwd_kernel(const
         compute_s(nx, (ST + 1) & 3, ka, st_next);
         compute_pv(ST, st);
         tc = nx;
-        __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
+        wait_vmcnt<4 * G::SPW>();
         barrier_lds_only();
     };
     // number of consecutive tiles from t on that are neither skipped nor masked
