@@ -275,6 +275,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // Consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
     // contiguous slice of the item list so that the q tiles of one (batch, head)
     // share that XCD's L2 copy of K/V.
+    // Fetch the launch parameters every path needs in one go: left alone, the compiler loads each
+    // field just before its first use, which puts a chain of dependent scalar-load round trips on the
+    // critical path of every workgroup.
+    asm volatile("" :: "s"(p.total_items), "s"(p.tiles_per_seq), "s"(p.H), "s"(p.M), "s"(p.N), "s"(p.nsplit),
+                 "s"(p.align_end), "s"(p.c1), "s"(p.cu_q), "s"(p.table), "s"(p.table_dtype));
+    asm volatile("" :: "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.q_sb), "s"(p.q_sh), "s"(p.q_sr),
+                 "s"(p.k_sb), "s"(p.k_sh), "s"(p.k_sr), "s"(p.v_sb), "s"(p.v_sh), "s"(p.v_sr));
+    asm volatile("" :: "s"(p.o_sb), "s"(p.o_sh), "s"(p.o_sr), "s"(p.t_sbucket), "s"(p.t_shead),
+                 "s"(p.bs.bidirectional), "s"(p.bs.nb), "s"(p.bs.max_exact), "s"(p.bs.n_thr), "s"(p.bs.sat));
     const int per_xcd = (p.total_items + 7) >> 3;
     int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (w >= p.total_items) return;
