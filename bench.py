@@ -280,7 +280,7 @@ def main():
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"dense bidirectional fused-bias attention forward, B{B} H{H} Lq=Lk={L} D{D} bf16, "
-                               "32 buckets max_distance 128, sm_scale 1.0 (BASELINE config 2)",
+                               "32 buckets max_distance 128, sm_scale 1.0 (baseline configuration 2)",
                    "device": props.name, "compute_units": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,

@@ -78,7 +78,7 @@ def test_dense_other_bucket_params(gpu_device):
 
 
 def test_config2_shape_subset(gpu_device):
-    """BASELINE config 2 (B16 H12 L1024 D64 bf16, N(0,1)*0.5, table N(0,1)); oracle on 2 batches."""
+    """Baseline configuration 2 (B16 H12 L1024 D64 bf16, N(0,1)*0.5, table N(0,1)); oracle on 2 batches."""
     from turbot5_amd.ops import flash_attention_with_fusing_bias
     g = torch.Generator().manual_seed(0)
     q, k, v = (0.5 * torch.randn(16, 12, 1024, 64, generator=g) for _ in range(3))

@@ -114,7 +114,7 @@ def test_bf16_attention_inside_fp32_model(gpu_device):
 
 
 def test_config1_t5_small_encoder(gpu_device):
-    """BASELINE config 1: T5-small random init (seed 0), batch 4 x 512 ids, all-ones mask, fp32."""
+    """Baseline configuration 1: T5-small random init (seed 0), batch 4 x 512 ids, all-ones mask, fp32."""
     cfg, m, sd = make(dict(vocab_size=32128, d_model=512, d_kv=64, d_ff=2048, num_layers=6, num_heads=8,
                            dropout_rate=0.0, attention_type="flash"), seed=0)
     ids = torch.randint(0, 32128, (4, 512), generator=torch.Generator().manual_seed(0))
