@@ -69,8 +69,30 @@ def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_dis
     return b, table   # keep `table` alive until the launch has been queued
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """hipStream_t of torch's current stream on t's device (the raw getter skips a Stream object per call)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device:
+    """Makes t's device current for the launch; a no-op (no context switch) when it already is."""
+
+    def __init__(self, t: torch.Tensor):
+        idx = t.device.index
+        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
 
 
 def _strides3(t):
@@ -94,7 +116,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
         raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
-    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
     o = torch.empty_like(q_)
     lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32) if return_lse else None
     a = L.T5ADenseArgs()
@@ -104,7 +126,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
     return (o, lse) if return_lse else o
 
@@ -134,7 +156,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
         sm_scale = 1.0 / math.sqrt(D)
     cq = cu_seqlens_q.to(device=q.device, dtype=torch.int32).contiguous()
     ck = cq if cu_seqlens_k is cu_seqlens_q else cu_seqlens_k.to(device=q.device, dtype=torch.int32).contiguous()
-    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
     lens = []
     for t in (seq_lens_q, seq_lens_k):
         if t is not None:
@@ -160,7 +182,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         L.check(L.load().t5a_fwd_varlen(C.byref(a), _stream(q)))
     return (o, lse) if return_lse else o
 
@@ -171,7 +193,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     B, H, Lq, D = q.shape
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("sparse self-attention needs q, k, v of one shape")
-    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
     o = torch.empty_like(q_)
     a = L.T5ASparseArgs()
     a.q, a.k, a.v, a.o = q_.data_ptr(), k_.data_ptr(), v_.data_ptr(), o.data_ptr()
@@ -197,7 +219,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     if ws_bytes > 0 and key_splits:   # block pattern: key splits of the global rows
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         a.workspace, a.workspace_bytes = workspace.data_ptr(), ws_bytes
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         L.check(lib.t5a_fwd_sparse(C.byref(a), _stream(q)))
     return o
 
@@ -264,7 +286,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     a.x_strides = (C.c_int64 * 2)(*strides)
     a.batches, a.rows_per_batch, a.dim, a.group = batches, rows, d, int(group)
     a.x_dtype, a.weight_dtype, a.eps = _dtype_code(x2), _dtype_code(w), float(eps)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         L.check(L.load().t5a_rmsnorm(C.byref(a), _stream(x)))
     return y
 
@@ -306,7 +328,7 @@ def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype):
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
     S = int(num_splits) if num_splits else default_num_splits(B, H, N, q.device)
-    q_, k_, v_ = (_kernel_ready(t.detach()) for t in (q, k, v))
+    q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
     lib = L.load()
     nbytes = lib.t5a_splitk_workspace_bytes(B, H, M, D, S)
     ws = torch.empty(max(nbytes, 16) // 4, device=q.device, dtype=torch.float32)
@@ -322,7 +344,7 @@ def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype):
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.num_splits, a.sm_scale = S, float(sm_scale)
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         L.check(lib.t5a_fwd_splitk(C.byref(a), _stream(q)))
     rows = B * H * S * M
     part_l = ws[rows * D: rows * D + rows].view(B, H, S, M)
