@@ -26,6 +26,13 @@ template <> struct SkLoad<__bf16> {
             out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
         }
     }
+    static __device__ __forceinline__ void widen(const unsigned __attribute__((ext_vector_type(4))) r, float* out) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[2 * i] = __uint_as_float(r[i] << 16);
+            out[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+        }
+    }
     static __device__ __forceinline__ __bf16 cvt(float x) { return static_cast<__bf16>(x); }
 };
 template <> struct SkLoad<_Float16> {
@@ -36,6 +43,12 @@ template <> struct SkLoad<_Float16> {
 #pragma unroll
         for (int i = 0; i < 8; ++i) out[i] = static_cast<float>(r[i]);
     }
+    static __device__ __forceinline__ void widen(const unsigned __attribute__((ext_vector_type(4))) r, float* out) {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        const h8 h = __builtin_bit_cast(h8, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = static_cast<float>(h[i]);
+    }
     static __device__ __forceinline__ _Float16 cvt(float x) { return static_cast<_Float16>(x); }
 };
 template <> struct SkLoad<float> {
@@ -43,6 +56,10 @@ template <> struct SkLoad<float> {
     static __device__ __forceinline__ void load(const float* p, float* out) {
         const float4 r = *reinterpret_cast<const float4*>(p);
         out[0] = r.x; out[1] = r.y; out[2] = r.z; out[3] = r.w;
+    }
+    static __device__ __forceinline__ void widen(const unsigned __attribute__((ext_vector_type(4))) r, float* out) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = __uint_as_float(r[i]);
     }
     static __device__ __forceinline__ float cvt(float x) { return x; }
 };
@@ -91,16 +108,31 @@ __global__ __launch_bounds__(SK_THREADS) void splitk_partial_kernel(const SplitK
         for (int x = 0; x < EPL; ++x) acc[m][x] = 0.f;
     }
 
-    for (int j0 = lo + slot; j0 < hi; j0 += KPP * UNROLL) {
-        float kf[UNROLL][EPL], vf[UNROLL][EPL];
+    // The loads of the next group of keys are in flight while the current group is reduced: the raw
+    // 16-byte words wait in registers and are widened to fp32 only when consumed.
+    typedef unsigned raw4 __attribute__((ext_vector_type(4)));
+    raw4 kraw[UNROLL], vraw[UNROLL];
+    auto fetch = [&](int j0) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int j = j0 + u * KPP;
             if (j < hi) {
-                L::load(kp + (int64_t)j * p.k_sr, kf[u]);
-                L::load(vp + (int64_t)j * p.v_sr, vf[u]);
+                kraw[u] = *reinterpret_cast<const raw4*>(kp + (int64_t)j * p.k_sr);
+                vraw[u] = *reinterpret_cast<const raw4*>(vp + (int64_t)j * p.v_sr);
             }
         }
+    };
+    if (lo + slot < hi) fetch(lo + slot);
+    for (int j0 = lo + slot; j0 < hi; j0 += KPP * UNROLL) {
+        float kf[UNROLL][EPL], vf[UNROLL][EPL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (j0 + u * KPP < hi) {
+                L::widen(kraw[u], kf[u]);
+                L::widen(vraw[u], vf[u]);
+            }
+        }
+        if (j0 + KPP * UNROLL < hi) fetch(j0 + KPP * UNROLL);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int j = j0 + u * KPP;
