@@ -184,3 +184,33 @@ def test_varlen_cross_lengths(gpu_device):
                                                       max(lq), max(lk), causal=causal, sm_scale=1.0)
         want = O.varlen_attention(q, k, v, table, cq, ck, causal, 1.0)
         assert (out.float().cpu() - want).abs().max().item() <= 2e-2
+
+
+def test_dense_on_a_side_stream_and_under_graph_capture(gpu_device):
+    """The library launches on the stream it is handed, allocates nothing and never synchronises: the op can
+    run on a non-default stream and be captured into a device graph.  Every replay (with fresh inputs copied
+    into the captured buffers, eager work and synchronisations in between) must equal the eager result."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    B, H, L, D = 2, 3, 384, 64
+    table = rnd(32, H, seed=203, scale=1.0).to(gpu_device)
+    sq, sk, sv = (torch.zeros(B, H, L, D, dtype=torch.bfloat16, device=gpu_device) for _ in range(3))
+    side = torch.cuda.Stream(device=gpu_device)
+    side.wait_stream(torch.cuda.current_stream(gpu_device))
+    with torch.cuda.stream(side):
+        for _ in range(3):                                   # warm-up outside the capture
+            flash_attention_with_fusing_bias(sq, sk, sv, table, causal=True, sm_scale=1.0)
+    torch.cuda.current_stream(gpu_device).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = flash_attention_with_fusing_bias(sq, sk, sv, table, causal=True, sm_scale=1.0)
+    for rep in range(4):
+        q, k, v = (rnd(B, H, L, D, seed=210 + 3 * rep + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+        eager = flash_attention_with_fusing_bias(q, k, v, table, causal=True, sm_scale=1.0)
+        torch.cuda.synchronize()
+        sq.copy_(q); sk.copy_(k); sv.copy_(v)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {rep} differs from the eager launch"
+    want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), table.cpu(), True, 1.0)
+    assert (captured.float().cpu() - want).abs().max().item() <= 2e-2
