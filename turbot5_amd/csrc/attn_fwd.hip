@@ -464,12 +464,19 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     auto cursor_dma = [&](int kstage, int vstage) {
         if constexpr (DMA) {
             const unsigned wbase = lds_base + (unsigned)wave * (1024u * G::SPW);
+            if constexpr (G::SPW == 1) {   // one request per tensor and wavefront
+                const u32x4 kr = {(unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0), 0x00020000u};
+                const u32x4 vr = {(unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0), 0x00020000u};
+                lds_dma_16(kr, wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES, cur_koff[0]);
+                lds_dma_16(vr, wbase + (unsigned)(vstage * V_TILE) * ES, cur_voff[0]);
+            } else {
 #pragma unroll
-            for (int c = 0; c < G::SPW; c += 2) {
-                lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
-                             wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES + c * 1024u, cur_koff[c], cur_koff[c + 1]);
-                lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
-                             wbase + (unsigned)(vstage * V_TILE) * ES + c * 1024u, cur_voff[c], cur_voff[c + 1]);
+                for (int c = 0; c + 1 < G::SPW; c += 2) {
+                    lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
+                                 wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES + c * 1024u, cur_koff[c], cur_koff[c + 1]);
+                    lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
+                                 wbase + (unsigned)(vstage * V_TILE) * ES + c * 1024u, cur_voff[c], cur_voff[c + 1]);
+                }
             }
             kcur += (unsigned)kstep; vcur += (unsigned)vstep;
             kleft -= kstep; vleft -= vstep;
