@@ -849,10 +849,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int x = 0; x < 4; ++x) pm[c] = max_ieee(pm[c], st[nt][4 * c + x]);
-        float mx = xhalf_max(max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3])));
-        const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
-        if (__any(raise)) {
+        // this lane's half of the row's keys; the other half sits in lane ^ 32 and is only consulted in the
+        // rare block: "some lane of the wavefront must raise" is the same question for halves and for rows
+        const float mh = max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3]));
+        if (__any((mh > kRaise) || (!started && mh > -INFINITY))) {
             asm volatile("");   // keep this rare block a real branch
+            const float mx = xhalf_max(mh);
+            const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
             const float delta = raise ? mx : 0.f;
             const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
             m_run += delta;
