@@ -3,7 +3,7 @@
 // One kernel template serves the dense, packed (cu_seqlens), local-window,
 // block+global and transient-global forwards.  A workgroup of four wavefronts
 // owns 128 query rows (32 per wavefront) of one (batch, head) and walks over
-// at most two key segments in tiles of 64 keys.  Per tile:
+// at most two key segments in tiles of 64 keys (32 at head_dim 128).  Per tile:
 //
 //   S^T = K Q^T + C  32x32 MFMA with K rows as the A operand, so that every
 //                    lane owns ONE query column and 16 keys per 32x32 block:
@@ -21,12 +21,17 @@
 //                    operand (for 16-bit types after a key permutation that is
 //                    baked into the LDS layout of V^T), so P stays in registers.
 //
-// 16-bit inputs (bf16, fp16) use v_mfma_f32_32x32x16; K tiles sit row-major in
-// LDS, V tiles transposed (head_dim x keys), both with an XOR swizzle on
-// 16-byte chunks.  fp32 inputs use v_mfma_f32_32x32x2_f32 (one float per lane
-// and operand) with K and V row-major and P kept in fp32.  Tiles are double
-// buffered and filled from registers that were loaded from HBM (buffer loads,
-// rows past the end of a segment read as zero) during the previous tile's math.
+// 16-bit inputs (bf16, fp16) use v_mfma_f32_32x32x16.  At head_dim 64 and 128
+// their K and V tiles are written into four-stage LDS rings by LDS-DMA buffer
+// loads (no staging registers; rows past the end of a segment arrive as
+// zeros), both row-major with an XOR swizzle on 16-byte chunks applied on the
+// source side, and V is transposed on the way out with ds_read_b64_tr_b16.
+// Other head dims stage through registers into double buffers, V transposed
+// on the LDS write.  fp32 inputs use v_mfma_f32_32x32x2_f32 (one float per
+// lane and operand) with K and V row-major and P kept in fp32.  The step for
+// tile t overlaps three things: the softmax head of tile t, the S product of
+// tile t+1 and the exp / PV product of tile t; runs of tiles that need neither
+// skipping nor masking take an unrolled fast path with compile-time stages.
 //
 // The T5 relative-position bias is not materialised.  Each workgroup expands
 // its head's column of the (num_buckets, H) table into a distance-indexed LUT
