@@ -257,7 +257,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     using v8 = typename E::v8;
     using v4 = typename E::v4;
     constexpr bool F32 = G::F32;
-    constexpr int EPC = G::EPC, KS = G::KS, DT = G::DT, VROWS = G::VROWS, CH = G::CH, SW = G::SW;
+    constexpr int KS = G::KS, DT = G::DT, VROWS = G::VROWS, CH = G::CH;
     constexpr int K_CHUNKS = G::K_CHUNKS, K_PER_T = G::K_PER_T, V_UNITS = G::V_UNITS, V_PER_T = G::V_PER_T;
     constexpr int KSTR = G::KSTR, K_TILE = G::K_TILE, V_TILE = G::V_TILE;
     constexpr int ES = sizeof(T);
