@@ -214,3 +214,35 @@ def test_dense_on_a_side_stream_and_under_graph_capture(gpu_device):
         assert torch.equal(captured, eager), f"replay {rep} differs from the eager launch"
     want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), table.cpu(), True, 1.0)
     assert (captured.float().cpu() - want).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("B,H,M,N", [(1, 12, 2048, 2048), (3, 5, 700, 700), (1, 1, 1500, 1500), (2, 3, 384, 1000),
+                                     (5, 7, 129, 129), (1, 12, 3000, 3000), (16, 12, 1024, 1024), (2, 3, 1000, 384)])
+def test_causal_item_order_writes_every_row(gpu_device, B, H, M, N):
+    """The causal launch cuts the item list into per-XCD slices of equal work and walks each slice longest
+    tile first; every (batch, head, tile) must still be computed exactly once.  Output and lse start as NaN
+    so that a tile nobody computed cannot pass by luck."""
+    import ctypes as C
+    from turbot5_amd import _lib as L
+    from turbot5_amd import ops
+    dt = torch.bfloat16
+    q, k, v = (rnd(B, H, n, 64, seed=40 + i, dtype=dt).to(gpu_device) for i, n in enumerate((M, N, N)))
+    table = rnd(32, H, seed=43, scale=1.0).to(gpu_device)
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, M), float("nan"), device=gpu_device, dtype=torch.float32)
+    a = L.T5ADenseArgs()
+    a.q, a.k, a.v, a.o, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr()
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = (ops._strides3(t) for t in (q, k, v, o))
+    a.dtype, a.B, a.H, a.M, a.N, a.D = L.T5A_BF16, B, H, M, N, 64
+    a.causal, a.sm_scale = 1, 1.0
+    a.bias, keep = ops._bias_struct(table, H, 32, 128, q)
+    L.check(L.load().t5a_fwd_dense(C.byref(a), ops._stream(q)))
+    torch.cuda.synchronize()
+    want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), table.cpu(), True, 1.0)
+    want_lse = O.dense_lse(q.cpu(), k.cpu(), table.cpu(), True, 1.0)
+    got = o.float().cpu()
+    assert not torch.isnan(got).any(), "rows left unwritten"
+    assert (got - want).abs().max().item() <= TOL[dt]
+    fin = torch.isfinite(want_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert (lse.cpu()[fin] - want_lse[fin]).abs().max().item() <= 2e-2

@@ -172,6 +172,35 @@ int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t
     return T5A_OK;
 }
 
+// Causal dense launch: cut the item list (pair-major, longest tile first inside a pair) into 8 slices of
+// equal work, one per XCD.  The cost of an item is its number of key tiles plus a constant for its
+// set-up and write-back (about five tile steps, from per-item timestamps).
+static void causal_slices(FwdParams* p, int dtype, int D) {
+    const int tps = p->tiles_per_seq;
+    const int bn = (dtype != T5A_F32 && D == 128) ? 32 : 64;   // keys per tile, as the kernel chooses them
+    const int64_t shift = (int64_t)p->N - p->M;                 // query i sits at key position i + N - M
+    auto cost = [&](int level) {                                // level 0 is the last (longest) q tile
+        const int64_t qt = tps - 1 - level;
+        const int64_t keys = std::min<int64_t>(p->N, std::max<int64_t>(0, (qt + 1) * 128 + shift));
+        return (keys + bn - 1) / bn + 5;
+    };
+    int64_t per_pair = 0;
+    for (int l = 0; l < tps; ++l) per_pair += cost(l);
+    const int64_t pairs = (int64_t)p->H * p->B;
+    const int64_t total = per_pair * pairs;
+    p->xcd_lo[0] = 0;
+    for (int x = 1; x < 8; ++x) {
+        const int64_t target = total * x / 8;
+        const int64_t g = target / per_pair;
+        int64_t rem = target - g * per_pair;
+        int l = 0;
+        while (l < tps && rem >= cost(l)) { rem -= cost(l); ++l; }
+        if (l < tps && 2 * rem > cost(l)) ++l;                  // nearer boundary
+        p->xcd_lo[x] = (int)std::min<int64_t>(g * tps + l, (int64_t)p->total_items);
+    }
+    p->xcd_lo[8] = p->total_items;
+}
+
 int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
@@ -201,6 +230,7 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     const int64_t items = (int64_t)p.tiles_per_seq * a->H * a->B;
     if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
     p.total_items = (int)items;
+    if (a->causal != 0 && p.tiles_per_seq > 1) causal_slices(&p, a->dtype, a->D);
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");

@@ -289,9 +289,24 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
                  "s"(p.k_sb), "s"(p.k_sh), "s"(p.k_sr), "s"(p.v_sb), "s"(p.v_sh), "s"(p.v_sr));
     asm volatile("" :: "s"(p.o_sb), "s"(p.o_sh), "s"(p.o_sr), "s"(p.t_sbucket), "s"(p.t_shead),
                  "s"(p.bs.bidirectional), "s"(p.bs.nb), "s"(p.bs.max_exact), "s"(p.bs.n_thr), "s"(p.bs.sat));
-    const int per_xcd = (p.total_items + 7) >> 3;
-    int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= p.total_items) return;
+    int w;
+    if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
+        // this XCD's slice [lo, hi) of the pair-major item list touches the pairs ga .. gb; walk that
+        // rectangle level by level (level 0 = longest tile) and drop the cells outside the slice
+        const unsigned x = blockIdx.x & 7, k = blockIdx.x >> 3;
+        const unsigned lo = (unsigned)p.xcd_lo[x], hi = (unsigned)p.xcd_lo[x + 1], tps = (unsigned)p.tiles_per_seq;
+        if (hi <= lo) return;
+        const unsigned ga = lo / tps, gx = (hi - 1) / tps - ga + 1;
+        if (k >= gx * tps) return;
+        const unsigned level = k / gx;
+        const unsigned wi = (ga + (k - level * gx)) * tps + level;
+        if (wi < lo || wi >= hi) return;
+        w = (int)wi;
+    } else {
+        const int per_xcd = (p.total_items + 7) >> 3;
+        w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if (w >= p.total_items) return;
+    }
 
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     int64_t q_off, k_off, v_off, o_off, lse_off;
@@ -1134,7 +1149,14 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
         if (e != hipSuccess) return e;
         granted.store(smem, std::memory_order_relaxed);
     }
-    const unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
+    unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
+    if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
+        unsigned most = 0;
+        for (int x = 0; x < 8; ++x)
+            if (p.xcd_lo[x + 1] > p.xcd_lo[x])
+                most = std::max(most, (unsigned)((p.xcd_lo[x + 1] - 1) / p.tiles_per_seq - p.xcd_lo[x] / p.tiles_per_seq + 1));
+        grid = 8u * most * (unsigned)p.tiles_per_seq;
+    }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
 }

@@ -39,6 +39,11 @@ struct FwdParams {
     int B, H, M, N;
     int tiles_per_seq;   // q tiles per (batch, head) when not packed
     int total_items;     // number of (q tile, head, batch) work items (upper bound when packed)
+    // causal, unpacked, no key split (xcd_lo[8] > 0): items shrink with the tile index, so the list (pair-major,
+    // longest tile first inside a (batch, head) pair) is cut into 8 slices of equal WORK, xcd_lo[x] .. xcd_lo[x+1]
+    // for XCD x, and an XCD visits its slice level by level: the longest tiles of all its pairs first, so that
+    // the kernel's tail is made of short items
+    int xcd_lo[9];
     float c1;            // sm_scale * log2(e)
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;
     int block_len, aux, n_side;
