@@ -112,17 +112,33 @@ int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
  * lens = mask.sum(-1), without the gathers and the scatter of the reference's unpad / pad
  * (src/turbot5/model/padding.py:113-150, :30-44).
  * lse (optional) is (total_q,H) contiguous fp32.
+ * workspace (optional): t5a_varlen_workspace_bytes(B, H, total_q) bytes of 16-byte aligned device
+ * memory (the function returns 0 when no plan can be made: B > 1024; a workspace is then
+ * ignored).  With it a one-workgroup kernel first builds a launch plan from
+ * cu_seqlens -- per-XCD item lists of equal WORK, longest item first -- on the same stream, still
+ * without host synchronisation; without it workgroups find their item by walking cu_seqlens and
+ * XCDs get equal item COUNTS, which leaves them unevenly loaded when lengths differ.  Results are
+ * identical either way.  Building the plan takes about 15 us on top of the launch: it pays from a
+ * few thousand q tiles x heads on, earlier when several calls share it (workspace_ready).  The
+ * workspace may be reused or freed once later work on the stream
+ * cannot overlap this call (stream order).
+ * workspace_ready != 0: the workspace still holds the plan that an earlier call built from the same
+ * cu_seqlens, seq_lens, B, H, D, dtype, causal and max_seqlen values (for instance the previous
+ * layer of the same batch): the build is skipped.
  */
 typedef struct t5a_varlen_args {
     const void* q; const void* k; const void* v; void* o; float* lse;
     int64_t q_strides[2]; int64_t k_strides[2]; int64_t v_strides[2]; int64_t o_strides[2];
     const int32_t* cu_seqlens_q; const int32_t* cu_seqlens_k;
     const int32_t* seq_lens_q; const int32_t* seq_lens_k;
+    void* workspace; int64_t workspace_bytes;
     int32_t dtype; int32_t B; int32_t H; int32_t D;
     int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
     int32_t causal; float sm_scale;
+    int32_t workspace_ready; int32_t reserved;
     t5a_bias bias;
 } t5a_varlen_args;
+int64_t t5a_varlen_workspace_bytes(int32_t B, int32_t H, int32_t total_q);
 int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
 
 /*

@@ -246,3 +246,110 @@ def test_causal_item_order_writes_every_row(gpu_device, B, H, M, N):
     fin = torch.isfinite(want_lse)
     assert torch.equal(torch.isfinite(lse.cpu()), fin)
     assert (lse.cpu()[fin] - want_lse[fin]).abs().max().item() <= 2e-2
+
+
+def _plan_case(name):
+    g = torch.Generator().manual_seed(11)
+    if name == "mixed":            # lengths as a tokenised batch has them, one empty sequence
+        lq = torch.randint(1, 1500, (40,), generator=g).tolist()
+        lq[7] = 0
+        return lq, lq
+    if name == "spill":            # a few long and many short sequences: the XCDs that take the short ones
+        lq = [4000] * 3 + [100] * 300   # hold far more items than their share of slots
+        return lq, lq
+    if name == "cross":            # keys longer than queries (cache), and shorter
+        lq = torch.randint(1, 1100, (64,), generator=g).tolist()
+        lk = [max(1, n + int(d)) for n, d in zip(lq, torch.randint(-300, 600, (64,), generator=g).tolist())]
+        return lq, lk
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", ["mixed", "spill", "cross"])
+def test_varlen_launch_plan(gpu_device, case, causal):
+    """Larger packed launches run from a device-built plan (per-XCD item lists of equal work).  The plan only
+    reorders items: the result equals, bit for bit, the one of the launch that walks cu_seqlens, and both
+    match the oracle.  The planned launch runs first, so memory left by the other cannot stand in for it."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    H, D = 4, 64
+    lq, lk = _plan_case(case)
+    cq = torch.tensor([0] + list(np.cumsum(lq)), dtype=torch.int32)
+    ck = torch.tensor([0] + list(np.cumsum(lk)), dtype=torch.int32)
+    q = rnd(int(cq[-1]), H, D, seed=50, dtype=torch.bfloat16)
+    k = rnd(int(ck[-1]), H, D, seed=51, dtype=torch.bfloat16)
+    v = rnd(int(ck[-1]), H, D, seed=52, dtype=torch.bfloat16)
+    table = rnd(32, H, seed=53, scale=1.0)
+    dev = [t.to(gpu_device) for t in (q, k, v, table, cq, ck)]
+    outs = []
+    for plan in ("always", False):
+        o, lse = flash_attention_with_fusing_bias_varlen(*dev, max(lq), max(lk), causal=causal, sm_scale=1.0,
+                                                         return_lse=True, launch_plan=plan)
+        torch.cuda.synchronize()
+        outs.append((o.cpu(), lse.cpu()))
+    assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16))
+    assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32))
+    want = O.varlen_attention(q, k, v, table, cq, ck, causal, 1.0)
+    assert (outs[0][0].float() - want).abs().max().item() <= 2e-2
+
+
+def test_varlen_launch_plan_with_padding_rows(gpu_device):
+    """planned launch over a right-padded batch given as cu = b * L plus lengths"""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    B, Lp, H, D = 24, 1024, 6, 64
+    lens = torch.randint(0, Lp + 1, (B,), generator=torch.Generator().manual_seed(12)).tolist()
+    lens[3] = Lp
+    q, k, v = (rnd(B * Lp, H, D, seed=60 + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+    table = rnd(32, H, seed=63, scale=1.0).to(gpu_device)
+    cu = torch.arange(0, (B + 1) * Lp, Lp, dtype=torch.int32, device=gpu_device)
+    ln = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    outs = [flash_attention_with_fusing_bias_varlen(q, k, v, table, cu, cu, Lp, Lp, causal=False, sm_scale=1.0,
+                                                    seq_lens_q=ln, seq_lens_k=ln, launch_plan=plan).cpu()
+            for plan in ("always", False)]
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    o = outs[0].view(B, Lp, H, D)
+    for b, n in enumerate(lens):
+        assert (o[b, n:] == 0).all()
+    b = 3
+    want = O.dense_attention(*(t.view(B, Lp, H, D)[b:b + 1].transpose(1, 2).cpu() for t in (q, k, v)), table.cpu(), False, 1.0)
+    assert (o[b:b + 1].transpose(1, 2).float() - want).abs().max().item() <= 2e-2
+
+
+def test_launch_plan_object_is_reused_and_rebuilt(gpu_device):
+    """One LaunchPlan over several calls: built by the first, found ready by the next (other q/k/v, same
+    lengths), rebuilt when the lengths are another tensor.  Every result equals the unplanned launch."""
+    from turbot5_amd.ops import LaunchPlan, flash_attention_with_fusing_bias_varlen
+    H, D = 4, 64
+    table = rnd(32, H, seed=73, scale=1.0).to(gpu_device)
+    plan = LaunchPlan()
+    g = torch.Generator().manual_seed(13)
+    built = []
+    for step, seed in enumerate((70, 71, 72)):
+        if step != 1:   # step 1 keeps the tensors of step 0
+            lens = torch.randint(600, 1400, (48,), generator=g).tolist()   # enough tiles for a plan
+            cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=gpu_device)
+        q, k, v = (rnd(int(cu[-1]), H, D, seed=seed + 10 * i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+        key_before = plan.key
+        got = flash_attention_with_fusing_bias_varlen(q, k, v, table, cu, cu, max(lens), max(lens), causal=True,
+                                                      sm_scale=1.0, launch_plan=plan)
+        built.append(plan.key != key_before)
+        want = flash_attention_with_fusing_bias_varlen(q, k, v, table, cu, cu, max(lens), max(lens), causal=True,
+                                                       sm_scale=1.0, launch_plan=False)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), step
+    assert built == [True, False, True]
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("lens", [[5, 128, 0, 129, 300, 1, 64], [700], [0, 0, 3], [129] * 9, [1] * 40])
+def test_launch_plan_of_tiny_batches(gpu_device, lens, causal):
+    """plans of a handful of items: empty sequences, one sequence, fewer items than XCDs"""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias_varlen
+    H, D = 3, 64
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    q, k, v = (rnd(int(cu[-1]), H, D, seed=80 + i, dtype=torch.bfloat16) for i in range(3))
+    table = rnd(32, H, seed=83, scale=1.0)
+    out = flash_attention_with_fusing_bias_varlen(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device),
+                                                  table.to(gpu_device), cu.to(gpu_device), cu.to(gpu_device),
+                                                  max(lens), max(lens), causal=causal, sm_scale=1.0,
+                                                  launch_plan="always")
+    want = O.varlen_attention(q, k, v, table, cu, cu, causal, 1.0)
+    assert (out.float().cpu() - want).abs().max().item() <= 2e-2

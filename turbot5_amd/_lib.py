@@ -17,6 +17,7 @@ PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
+    "t5a_varlen_workspace_bytes",
     "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_rmsnorm",
 )
 
@@ -42,9 +43,11 @@ class T5AVarlenArgs(C.Structure):
                 ("o_strides", C.c_int64 * 2),
                 ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
                 ("seq_lens_q", C.c_void_p), ("seq_lens_k", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32),
                 ("max_seqlen_k", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
+                ("workspace_ready", C.c_int32), ("reserved", C.c_int32),
                 ("bias", T5ABias)]
 
 
@@ -112,6 +115,8 @@ def load() -> C.CDLL:
         lib.t5a_splitk_workspace_bytes.restype = C.c_int64
         lib.t5a_rmsnorm.argtypes = [C.POINTER(T5ARmsNormArgs), C.c_void_p]
         lib.t5a_rmsnorm.restype = C.c_int
+        lib.t5a_varlen_workspace_bytes.argtypes = [C.c_int32] * 3
+        lib.t5a_varlen_workspace_bytes.restype = C.c_int64
         lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7
         lib.t5a_sparse_workspace_bytes.restype = C.c_int64
         _lib = lib

@@ -84,8 +84,15 @@ def _mask_info(mask: torch.Tensor):
         [valid.all(), (valid == (steps[None, :] < lens[:, None])).all()]).tolist())
     unpad = None
     if not all_ones:
-        # right-padded batches run in place with per-sequence lengths; anything else is packed first
-        unpad = ("lens", lens) if right_padded else ("packed", _get_unpad_data(valid.to(torch.int32)))
+        # right-padded batches run in place with per-sequence lengths; anything else is packed first.
+        # The last element collects the launch plans of this batch, one per kind of attention call, so
+        # that the layers of a stack build each only once.
+        if right_padded:
+            B, L = mask.shape
+            cu = torch.arange(0, (B + 1) * L, L, dtype=torch.int32, device=mask.device)
+            unpad = ("lens", (lens, cu), {})
+        else:
+            unpad = ("packed", _get_unpad_data(valid.to(torch.int32)), {})
     _MASK_INFO[key] = (all_ones, unpad)
     while len(_MASK_INFO) > 16:
         _MASK_INFO.popitem(last=False)
@@ -200,22 +207,29 @@ class T5FlashAttention(_T5AttentionBase):
             q_blhd = query_states.transpose(1, 2)
             k_blhd = key_states.transpose(1, 2)
             v_blhd = value_states.transpose(1, 2)
-            kind, unpad = unpad
+            kind, unpad, plans = unpad
             dev = hidden_states.device
+            # self-attention over the batch: cu_seqlens come from the per-mask cache, so the layers can share
+            # one plan; other calls make their cu_q on the spot and plan per call
+            plan = True
+            if key_value_states is None and seq_length == key_length:
+                plan = plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt, seq_length),
+                                        ops.LaunchPlan())
             if kind == "lens":
                 # right-padded batch: the kernel walks the padded (B*L, H, D) layout with per-sequence
                 # lengths; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
                 def rows(t, n):
                     t = t if t.is_contiguous() else t.contiguous()
                     return t.view(batch_size * n, self.n_heads, -1)
-                cu_k = torch.arange(0, (batch_size + 1) * key_length, key_length, dtype=torch.int32, device=dev)
+                unpad, cu_k = unpad
                 self_attn = key_value_states is None and seq_length == key_length
                 cu_q = cu_k if self_attn else torch.arange(0, (batch_size + 1) * seq_length, seq_length,
                                                            dtype=torch.int32, device=dev)
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
                     rows(q_blhd, seq_length), rows(k_blhd, key_length), rows(v_blhd, key_length), table, cu_q, cu_k,
                     seq_length, key_length, causal=self.causal, sm_scale=1.0, NUM_BUCKETS=nb, MAX_DISTANCE=md,
-                    seq_lens_q=unpad if self_attn else None, seq_lens_k=unpad)
+                    seq_lens_q=unpad if self_attn else None, seq_lens_k=unpad,
+                    launch_plan=plan)
                 attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
             elif key_value_states is None and seq_length == key_length:
                 q_p, k_p, v_p, indices_q, (cu_q, cu_k), (max_q, max_k) = _upad_input(
@@ -232,7 +246,7 @@ class T5FlashAttention(_T5AttentionBase):
             if kind != "lens":
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
                     q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
-                    NUM_BUCKETS=nb, MAX_DISTANCE=md)
+                    NUM_BUCKETS=nb, MAX_DISTANCE=md, launch_plan=plan)
                 if indices_q is not None:
                     attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
                 else:

@@ -236,6 +236,17 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
 }
 
+// Entries per XCD of a packed batch's launch plan: twice the mean, so that slices of equal work but
+// unequal item counts fit (a slice that still outgrows it spills into the others' free slots).
+static int plan_slots(int64_t items_bound) { return (int)(2 * ((items_bound + 7) / 8)); }
+
+int64_t t5a_varlen_workspace_bytes(int32_t B, int32_t H, int32_t total_q) {
+    if (B <= 0 || H <= 0 || total_q <= 0 || B > kPlanMaxSeqs) return 0;
+    const int64_t items = ((int64_t)total_q / 128 + B) * H;
+    if (items > 0x03ffff00LL) return 0;
+    return 64 + (int64_t)8 * plan_slots(items) * 32 + items * 16;   // counts, the lists, room for spilled items
+}
+
 int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
@@ -272,6 +283,34 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     p.align_end = 1;
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
+    const int64_t need = t5a_varlen_workspace_bytes(a->B, a->H, a->total_q);
+    if (a->workspace != nullptr && need > 0) {
+        // launch plan: per-XCD item lists of equal work, longest first, built on the device
+        if (a->workspace_bytes < need)
+            return fail(T5A_ERR_WORKSPACE, "workspace too small: %lld bytes, t5a_varlen_workspace_bytes() asks for %lld",
+                        (long long)a->workspace_bytes, (long long)need);
+        if ((reinterpret_cast<uintptr_t>(a->workspace) & 15) != 0)
+            return fail(T5A_ERR_STRIDE, "workspace must be 16-byte aligned");
+        PlanParams pl;
+        memset(&pl, 0, sizeof(pl));
+        pl.cu_q = a->cu_seqlens_q; pl.cu_k = a->cu_seqlens_k; pl.len_q = a->seq_lens_q; pl.len_k = a->seq_lens_k;
+        pl.B = a->B; pl.H = a->H; pl.causal = a->causal != 0;
+        pl.bn_shift = (a->dtype != T5A_F32 && a->D == 128) ? 5 : 6;
+        const int max_cost = (a->max_seqlen_k >> pl.bn_shift) + 8;
+        while ((max_cost >> pl.key_shift) >= 512) ++pl.key_shift;
+        pl.slots = plan_slots(items);
+        pl.staged = plan_can_stage(pl.slots, a->H, a->max_seqlen_q) ? 1 : 0;
+        pl.counts = static_cast<int32_t*>(a->workspace);
+        pl.plan = pl.counts + 16;
+        pl.spill = pl.plan + (size_t)8 * pl.slots * 8;
+        if (a->workspace_ready == 0) {
+            hipError_t e = launch_varlen_plan(pl, (hipStream_t)stream);
+            if (e != hipSuccess) return finish(e, "t5a_fwd_varlen (plan)");
+        }
+        p.plan = pl.plan;
+        p.plan_counts = pl.counts;
+        p.plan_slots = pl.slots;
+    }
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
 }
 

@@ -284,13 +284,16 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // field just before its first use, which puts a chain of dependent scalar-load round trips on the
     // critical path of every workgroup.
     asm volatile("" :: "s"(p.total_items), "s"(p.tiles_per_seq), "s"(p.H), "s"(p.M), "s"(p.N), "s"(p.nsplit),
-                 "s"(p.align_end), "s"(p.c1), "s"(p.cu_q), "s"(p.table), "s"(p.table_dtype));
+                 "s"(p.align_end), "s"(p.c1), "s"(p.cu_q), "s"(p.plan), "s"(p.table), "s"(p.table_dtype));
     asm volatile("" :: "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.q_sb), "s"(p.q_sh), "s"(p.q_sr),
                  "s"(p.k_sb), "s"(p.k_sh), "s"(p.k_sr), "s"(p.v_sb), "s"(p.v_sh), "s"(p.v_sr));
     asm volatile("" :: "s"(p.o_sb), "s"(p.o_sh), "s"(p.o_sr), "s"(p.t_sbucket), "s"(p.t_shead),
                  "s"(p.bs.bidirectional), "s"(p.bs.nb), "s"(p.bs.max_exact), "s"(p.bs.n_thr), "s"(p.bs.sat));
-    int w;
-    if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
+    int w = 0;
+    const bool planned = MODE == kDense && p.plan != nullptr;
+    if (planned) {
+        // the item comes from the launch plan, below
+    } else if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
         // this XCD's slice [lo, hi) of the pair-major item list touches the pairs ga .. gb; walk that
         // rectangle level by level (level 0 = longest tile) and drop the cells outside the slice
         const unsigned x = blockIdx.x & 7, k = blockIdx.x >> 3;
@@ -311,23 +314,32 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     int64_t q_off, k_off, v_off, o_off, lse_off;
     if (MODE == kDense && p.cu_q != nullptr) {
-        // packed batch: find (sequence, head, tile) by walking cu_seqlens
-        int acc = 0, nt_b = 0, qs = 0;
-        b = -1;
-        for (int bb = 0; bb < p.B; ++bb) {
-            qs = p.cu_q[bb];
-            const int len = p.len_q != nullptr ? p.len_q[bb] : p.cu_q[bb + 1] - qs;
-            nt_b = (len + BM - 1) / BM;
-            const int cnt = nt_b * p.H;
-            if (w < acc + cnt) { b = bb; Mseq = len; w -= acc; break; }
-            acc += cnt;
+        int qs = 0, ks = 0;
+        if (planned) {
+            // packed batch with a launch plan: entry k of this XCD's list
+            const int x = blockIdx.x & 7, k = blockIdx.x >> 3;
+            const int* e = p.plan + ((size_t)x * p.plan_slots + k) * 8;
+            if (k >= p.plan_counts[x]) return;
+            b = e[0]; h = e[1]; qt = e[2]; Mseq = e[3]; Nseq = e[4]; qs = e[5]; ks = e[6];
+        } else {
+            // packed batch: find (sequence, head, tile) by walking cu_seqlens
+            int acc = 0, nt_b = 0;
+            b = -1;
+            for (int bb = 0; bb < p.B; ++bb) {
+                qs = p.cu_q[bb];
+                const int len = p.len_q != nullptr ? p.len_q[bb] : p.cu_q[bb + 1] - qs;
+                nt_b = (len + BM - 1) / BM;
+                const int cnt = nt_b * p.H;
+                if (w < acc + cnt) { b = bb; Mseq = len; w -= acc; break; }
+                acc += cnt;
+            }
+            if (b < 0) return;
+            h = w / nt_b;
+            qt = w - h * nt_b;
+            if (CAUSAL) qt = nt_b - 1 - qt;
+            ks = p.cu_k[b];
+            Nseq = p.len_k != nullptr ? p.len_k[b] : p.cu_k[b + 1] - ks;
         }
-        if (b < 0) return;
-        h = w / nt_b;
-        qt = w - h * nt_b;
-        if (CAUSAL) qt = nt_b - 1 - qt;
-        const int ks = p.cu_k[b];
-        Nseq = p.len_k != nullptr ? p.len_k[b] : p.cu_k[b + 1] - ks;
         q_off = (int64_t)qs * p.q_sr + (int64_t)h * p.q_sh;
         o_off = (int64_t)qs * p.o_sr + (int64_t)h * p.o_sh;
         k_off = (int64_t)ks * p.k_sr + (int64_t)h * p.k_sh;
@@ -1150,6 +1162,7 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
         granted.store(smem, std::memory_order_relaxed);
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
+    if (MODE == kDense && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
     if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
         unsigned most = 0;
         for (int x = 0; x < 8; ++x)

@@ -36,6 +36,8 @@ struct FwdParams {
     int64_t lse_sb, lse_sh, lse_sr;
     const int32_t* cu_q; const int32_t* cu_k;   // non-null: packed variable-length batch
     const int32_t* len_q; const int32_t* len_k; // optional lengths (rows between cu[b]+len[b] and cu[b+1] are padding)
+    // packed batch with a launch plan (plan.hip): workgroup 8 k + x runs the item in plan[x][k]
+    const int32_t* plan; const int32_t* plan_counts; int plan_slots;
     int B, H, M, N;
     int tiles_per_seq;   // q tiles per (batch, head) when not packed
     int total_items;     // number of (q tile, head, batch) work items (upper bound when packed)
@@ -76,6 +78,23 @@ struct SplitKParams {
 hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t stream);
 // only the merge over splits (part_o, part_l, part_m -> o)
 hipError_t launch_splitk_merge(const SplitKParams& p, int dtype, int D, hipStream_t stream);
+
+// Launch plan of a packed batch: 8 lists (one per XCD) of `slots` entries of 8 ints
+// {sequence, head, q tile, len_q, len_k, first q row, first k row, 0}, of which the first counts[x] are in use.
+constexpr int kPlanMaxSeqs = 1024;
+struct PlanParams {
+    const int32_t* cu_q; const int32_t* cu_k; const int32_t* len_q; const int32_t* len_k;
+    int B, H, causal;
+    int bn_shift;    // log2(keys per tile) of the attention kernel that will run the plan
+    int key_shift;   // cost >> key_shift < 512 for every item
+    int slots;       // entries per XCD
+    int staged;      // 1: build the lists in LDS first (plan_can_stage() said they fit)
+    int32_t* counts; // [8]
+    int32_t* plan;   // [8][slots][8]
+    int32_t* spill;  // scratch: four ints per item
+};
+bool plan_can_stage(int slots, int H, int max_seqlen_q);
+hipError_t launch_varlen_plan(const PlanParams& p, hipStream_t stream);
 
 struct RmsParams {
     const void* x; const void* weight; void* y;

@@ -131,9 +131,40 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     return (o, lse) if return_lse else o
 
 
+PLAN_MIN_ITEMS = 3072          # (q tiles x heads) from which a launch plan is built for a single call
+PLAN_MIN_ITEMS_SHARED = 1024   # ... when a LaunchPlan object shares it between calls
+
+
+class LaunchPlan:
+    """Keeps the launch plan of one packed batch so that calls with the same lengths share it.
+
+    Pass one object as ``launch_plan=`` to every ``flash_attention_with_fusing_bias_varlen`` call over
+    the same batch (the layers of a stack): the first call builds the plan on the device, the others
+    find the workspace ready.  The object compares the identity and version of the length tensors
+    (int32 device tensors, which it keeps alive) and the launch shape, and rebuilds when they differ;
+    lengths changed behind torch's back (a raw kernel writing into the same tensor) go unnoticed.
+    Use one object per stream.
+    """
+
+    def __init__(self):
+        self.key = None
+        self.tensors = None     # the length tensors of the key, kept alive: their addresses cannot be reused
+        self.workspace = None
+
+    def lookup(self, key, tensors, nbytes, device):
+        """-> (workspace, ready)"""
+        if self.key == key and self.workspace is not None:
+            return self.workspace, True
+        if self.workspace is None or self.workspace.numel() < nbytes or self.workspace.device != device:
+            self.workspace = torch.empty(nbytes, device=device, dtype=torch.uint8)
+        self.key, self.tensors = key, tensors
+        return self.workspace, False
+
+
 def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                             causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                            return_lse: bool = False, seq_lens_q=None, seq_lens_k=None):
+                                            return_lse: bool = False, seq_lens_q=None, seq_lens_k=None,
+                                            launch_plan: bool = True):
     """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
 
     Positions restart at 0 in every sequence.  No host synchronisation: the
@@ -143,6 +174,11 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     [cu[b], cu[b] + lens[b]); the rows up to cu[b+1] are padding, never read and left ZERO in the
     output.  A right-padded (B, L, H, D) batch runs in place this way, viewed as (B*L, H, D) with
     cu = arange(B+1) * L and lens = mask.sum(-1): no gathers, no scatter.
+
+    ``launch_plan``: True (default) lets larger launches first build, on the device, per-XCD item
+    lists of equal work from ``cu_seqlens`` (a small workspace is taken from torch's allocator);
+    False never does, ``"always"`` does whatever the size.  A ``LaunchPlan`` object keeps the plan
+    for later calls over the same batch.  The results do not depend on any of this.
     """
     _check_inputs(q, k, v)
     total_q, H, D = q.shape
@@ -182,8 +218,24 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    lib = L.load()
+    # building a plan costs about 15 us: worth it from a few thousand items on, earlier when shared
+    items = (total_q // 128 + B) * H
+    shared = isinstance(launch_plan, LaunchPlan)
+    wanted = launch_plan == "always" or (shared and items >= PLAN_MIN_ITEMS_SHARED) or \
+        (launch_plan is True and items >= PLAN_MIN_ITEMS)
+    ws_bytes = lib.t5a_varlen_workspace_bytes(B, H, total_q) if wanted else 0
+    if ws_bytes > 0:
+        if isinstance(launch_plan, LaunchPlan):
+            key = tuple((t.data_ptr(), t._version) if t is not None else None for t in (cq, ck, lens[0], lens[1]))
+            key += (B, H, D, total_q, a.dtype, a.causal, a.max_seqlen_q, a.max_seqlen_k, str(q.device))
+            ws, ready = launch_plan.lookup(key, (cq, ck, lens[0], lens[1]), ws_bytes, q.device)
+            a.workspace_ready = int(ready)
+        else:
+            ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)   # stream-ordered reuse by torch's allocator
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
     with _on_device(q):
-        L.check(L.load().t5a_fwd_varlen(C.byref(a), _stream(q)))
+        L.check(lib.t5a_fwd_varlen(C.byref(a), _stream(q)))
     return (o, lse) if return_lse else o
 
 
