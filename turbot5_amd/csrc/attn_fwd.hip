@@ -137,6 +137,23 @@ __device__ __forceinline__ float load_table(const void* table, int dtype, int64_
     return static_cast<float>(reinterpret_cast<const _Float16*>(table)[off]);
 }
 
+// Table element fetched from inline assembly, so that the kernel decides how long to wait for it
+// (see the prologue): `raw` receives the element's bits, zero-extended for the 16-bit types.
+__device__ __forceinline__ void load_table_async(const void* table, int dtype, int64_t off, unsigned& raw) {
+    if (dtype == T5A_F32) {
+        const float* a = reinterpret_cast<const float*>(table) + off;
+        asm volatile("global_load_dword %0, %1, off" : "+v"(raw) : "v"(a) : "memory");
+    } else {
+        const unsigned short* a = reinterpret_cast<const unsigned short*>(table) + off;
+        asm volatile("global_load_ushort %0, %1, off" : "+v"(raw) : "v"(a) : "memory");
+    }
+}
+__device__ __forceinline__ float table_value(unsigned raw, int dtype) {
+    if (dtype == T5A_F32) return __uint_as_float(raw);
+    if (dtype == T5A_BF16) return __uint_as_float(raw << 16);
+    return static_cast<float>(__builtin_bit_cast(_Float16, (unsigned short)raw));
+}
+
 // max / sum over the two lanes (l, l^32) that share a query row; the swap
 // exchanges the upper half of one operand with the lower half of the other, so
 // combining both results is symmetric in the halves.
@@ -514,18 +531,6 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             kleft -= kstep; vleft -= vstep;
         }
     };
-    // request the first tiles right away: they arrive while the bias LUT and the Q fragments are set up
-    if constexpr (DMA) {
-        if constexpr (MODE == kDense) {
-            cursor_seek(0, 0);
-            cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
-            dma_tile(3, false);                                     // K3
-        } else {
-            for (int i = 0; i < 4; ++i) dma_tile(i, false);
-            for (int i = 0; i < 3; ++i) dma_tile(i, true);
-        }
-    }
-
     // ---------------------------------------------------------------- Q fragments: loads first
     const int iw0 = i0 + wave * 32;      // first row of this wavefront
     const int iw1 = iw0 + 31;
@@ -556,15 +561,33 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     const int quads = lut_quads(sat, CAUSAL);
     const int qlen = 4 * quads;
     const float log2e = 1.4426950408889634f;
+    // The head's table column: with at most 64 buckets, lane b of every wavefront fetches bucket b up
+    // front and the LUT entries pick their value with a lane permute; larger tables are read per entry.
+    // Order of the prologue's memory requests: Q rows, table column, then the first K/V tiles.  Loads
+    // complete in order, so "at most the tile requests outstanding" means Q and the column are here,
+    // and the LUT is built while the tiles are still in flight (built after a wait for everything,
+    // it made up half of the 5 us a work item spends outside its tile loop).
+    const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
+    const bool col_in_lanes = nbt <= 64;
+    unsigned tcol_raw = 0;
+    if (has_bias && col_in_lanes && lane < nbt)
+        load_table_async(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead, tcol_raw);
+    // request the first tiles: they arrive while the bias LUT is built
+    if constexpr (DMA) {
+        if constexpr (MODE == kDense) {
+            cursor_seek(0, 0);
+            cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
+            dma_tile(3, false);                                     // K3
+        } else {
+            for (int i = 0; i < 4; ++i) dma_tile(i, false);
+            for (int i = 0; i < 3; ++i) dma_tile(i, true);
+        }
+    }
+
+    constexpr int PROLOGUE_TILE_REQUESTS = DMA ? 7 * G::SPW : 0;   // per wavefront, all issued after the column load
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(tcol_raw) : "n"(PROLOGUE_TILE_REQUESTS));
     if (has_lut) {
-        // The head's table column: with at most 64 buckets, lane b of every wavefront fetches bucket b
-        // up front (independent of the bucket arithmetic) and the LUT entries pick their value with a
-        // lane permute; larger tables are read per entry.
-        const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
-        const bool col_in_lanes = nbt <= 64;
-        float tcol = 0.f;
-        if (has_bias && col_in_lanes && lane < nbt)
-            tcol = load_table(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+        const float tcol = table_value(tcol_raw, p.table_dtype) * log2e;
         // one evaluation per distance; the value goes to all four shifted copies:
         // copy a, slot i holds the distance i + a - padl
         for (int e0 = 0; e0 < qlen + 3; e0 += NTHREADS) {   // uniform trip count: the permute needs every lane
