@@ -98,6 +98,16 @@ def extra_workloads(torch, dev, steps, full):
             "total_tokens": tot, "ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
     del q, k, v
 
+    # ---- causal dense (decoder self-attention over a prompt): FLOPs of the visible pairs only
+    for bsz, ln in ((16, 1024), (4, 4096)):
+        q, k, v, table = make_inputs(torch, dev, bsz, H, ln, D, seed=7)
+        f = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=True, sm_scale=1.0)  # noqa: E731
+        _, ms = time_kernel(torch, f, reps, warm)
+        tf = 4.0 * bsz * H * D * (ln * (ln + 1) // 2) / (ms * 1e-3) / 1e12
+        out[f"dense_causal_B{bsz}_H{H}_L{ln}"] = {"ms": round(ms, 4), "tflops": round(tf, 1),
+                                                 "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+        del q, k, v
+
     # ---- head_dim 128 (the T5-3B / 11B head shape): B4 H6 L4096, same FLOPs as the B4 H12 D64 sweep point
     g = torch.Generator().manual_seed(6)
     q, k, v = ((0.5 * torch.randn(4, 6, 4096, 128, generator=g)).to(torch.bfloat16).to(dev) for _ in range(3))

@@ -311,7 +311,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
         p.plan_counts = pl.counts;
         p.plan_slots = pl.slots;
     }
-    return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
+    return finish(launch_fwd(p, a->dtype, a->D, kPacked, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
 }
 
 // Key splits for the global rows of the block pattern: enough (batch, head, split) items to fill the

@@ -279,6 +279,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     constexpr int KSTR = G::KSTR, K_TILE = G::K_TILE, V_TILE = G::V_TILE;
     constexpr int ES = sizeof(T);
     constexpr int BN = G::BN, NT = G::NT;
+    constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr bool DMA = G::DMA;
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     asm volatile("" :: "s"(p.o_sb), "s"(p.o_sh), "s"(p.o_sr), "s"(p.t_sbucket), "s"(p.t_shead),
                  "s"(p.bs.bidirectional), "s"(p.bs.nb), "s"(p.bs.max_exact), "s"(p.bs.n_thr), "s"(p.bs.sat));
     int w = 0;
-    const bool planned = MODE == kDense && p.plan != nullptr;
+    const bool planned = MODE == kPacked && p.plan != nullptr;
     if (planned) {
         // the item comes from the launch plan, below
     } else if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
 
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     int64_t q_off, k_off, v_off, o_off, lse_off;
-    if (MODE == kDense && p.cu_q != nullptr) {
+    if (MODE == kPacked) {
         int qs = 0, ks = 0;
         if (planned) {
             // packed batch with a launch plan: entry k of this XCD's list
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     seg_start[0] = 0; seg_end[0] = 0;
     seg_start[1] = seg_end[1] = seg_lend[1] = 0; seg_kind[1] = 0; seg_win[1] = 0;
     seg_kind[0] = 0; seg_win[0] = 0; seg_lend[0] = Nseq;
-    if (MODE == kDense) {
+    if (DENSE) {
         seg_end[0] = CAUSAL ? max(0, min(Nseq, i0 + BM + P)) : Nseq;
     } else if (MODE == kLocal || MODE == kTGlobal) {
         seg_start[0] = max(0, i0 - p.block_len + 1);
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     int cur_koff[G::SPW], cur_voff[G::SPW];
 #pragma unroll
     for (int c = 0; c < G::SPW; ++c) cur_koff[c] = cur_voff[c] = 0;
-    if constexpr (DMA && MODE == kDense) {
+    if constexpr (DMA && DENSE) {
 #pragma unroll
         for (int c = 0; c < G::SPW; ++c) {
             const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
@@ -574,7 +575,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         load_table_async(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead, tcol_raw);
     // request the first tiles: they arrive while the bias LUT is built
     if constexpr (DMA) {
-        if constexpr (MODE == kDense) {
+        if constexpr (DENSE) {
             cursor_seek(0, 0);
             cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
             dma_tile(3, false);                                     // K3
@@ -748,7 +749,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // dense / packed mode: one segment starting at key 0, so the class of tile t follows from four
     // per-wavefront thresholds
     int d_tl = 0, d_tr = 0, d_ts = 0, d_tm = 0;
-    if (MODE == kDense) {
+    if (DENSE) {
         const int qlo = iw0 + P, qhi = iw1 + P;
         const int lim = qlo - (BN - 1) - sat;                  // left-saturated tiles: BN*t <= lim
         d_tl = lim < 0 ? 0 : lim / BN + 1;
@@ -760,7 +761,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         TileClass c;
         c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
         if (t >= ntiles) return c;
-        if (MODE == kDense) {
+        if (DENSE) {
             c.j0 = t * BN;
             c.skip = t >= d_ts;
             const bool left_sat = t < d_tl, right_sat = t >= d_tr;
@@ -1070,7 +1071,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // compile time.
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
-        if constexpr (MODE == kDense) cursor_dma(ST, (ST + 3) & 3);
+        if constexpr (DENSE) cursor_dma(ST, (ST + 3) & 3);
         else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
@@ -1088,7 +1089,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     };
     // number of consecutive tiles from t on that are neither skipped nor masked
     auto plain_run = [&](int t) {
-        if (MODE == kDense) return max(0, min(min(d_ts, d_tm), ntiles) - t);
+        if (DENSE) return max(0, min(min(d_ts, d_tm), ntiles) - t);
         int n = 0;
         for (; t + n < ntiles; ++n) {
             const TileClass c = classify(t + n);
@@ -1107,7 +1108,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             int quads = (t + run >= ntiles ? run : run - 1) >> 2;
             if (quads > 0) {
                 tc = classify(t);
-                if constexpr (MODE == kDense) cursor_seek(t + 4, t + 3);
+                if constexpr (DENSE) cursor_seek(t + 4, t + 3);
             }
             while (quads > 0) {
                 fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
@@ -1185,7 +1186,7 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
         granted.store(smem, std::memory_order_relaxed);
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
-    if (MODE == kDense && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
+    if (MODE == kPacked && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
     if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
         unsigned most = 0;
         for (int x = 0; x < 8; ++x)
@@ -1201,6 +1202,7 @@ template <typename T, int D>
 static hipError_t launch_mode(const FwdParams& p, int mode, bool causal, hipStream_t s) {
     switch (mode) {
         case kDense: return causal ? launch_one<T, D, kDense, true>(p, s) : launch_one<T, D, kDense, false>(p, s);
+        case kPacked: return causal ? launch_one<T, D, kPacked, true>(p, s) : launch_one<T, D, kPacked, false>(p, s);
         case kLocal: return launch_one<T, D, kLocal, false>(p, s);
         case kBlock: return launch_one<T, D, kBlock, false>(p, s);
         case kTGlobal: return launch_one<T, D, kTGlobal, false>(p, s);

@@ -22,7 +22,9 @@ struct BucketSpec {
     int thr[kMaxThresholds];
 };
 
-enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3 };
+// kPacked: dense semantics per sequence of a packed batch (cu_seqlens); a separate instantiation, so that
+// the unpacked kernel carries none of its work-item search
+enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4 };
 
 struct FwdParams {
     const void* q; const void* k; const void* v; void* o; float* lse;
