@@ -56,16 +56,28 @@ typedef enum t5a_pattern {
     T5A_PATTERN_TGLOBAL = 3  /* sliding window + side tokens (one per aux block of tokens) */
 } t5a_pattern;
 
-/* The (num_buckets, H) relative-attention table (nn.Embedding weight).  table == NULL: no bias. */
+/*
+ * The (num_buckets, H) relative-attention table (nn.Embedding weight).  table == NULL: no bias.
+ * lut (optional): t5a_bias_lut_bytes() bytes of 16-byte aligned device memory.  Every work item of the
+ * attention kernels starts by expanding its head's table column into a bias-per-distance LUT; with this
+ * buffer the LUTs of all heads are built once (on the call's stream, by the first call: lut_ready == 0) and
+ * later calls fetch them (lut_ready != 0: the buffer holds the LUTs of the same table values, bucket
+ * parameters, H and causal flag).  Results are identical with and without it; it shortens the set-up of a
+ * work item (4 % of the run time at B16 H12 L1024 D64).  Rebuild after the table changes.
+ */
 typedef struct t5a_bias {
     const void* table;
     int32_t table_dtype;          /* T5A_F32, T5A_BF16 or T5A_F16 */
     int32_t num_buckets;
     int32_t max_distance;
-    int32_t reserved;
+    int32_t lut_ready;
     int64_t stride_bucket;        /* elements between buckets (torch stride(0)) */
     int64_t stride_head;          /* elements between heads   (torch stride(1)) */
+    void* lut; int64_t lut_bytes;
 } t5a_bias;
+/* 0 when the kernels cannot use a LUT buffer for these parameters (very large max_distance); causal selects
+ * the unidirectional buckets, as in t5a_fwd_dense. */
+int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t causal);
 
 int t5a_version(void);
 const char* t5a_last_error(void);

@@ -353,3 +353,61 @@ def test_launch_plan_of_tiny_batches(gpu_device, lens, causal):
                                                   launch_plan="always")
     want = O.varlen_attention(q, k, v, table, cu, cu, causal, 1.0)
     assert (out.float().cpu() - want).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_bias_lut_buffer_gives_identical_results(gpu_device, causal):
+    """The LUTs of all heads, built once into a buffer and fetched by later launches, are the image a work item
+    otherwise builds for itself: outputs are bit-identical with and without the buffer, on the launch that
+    builds it and on the ones that find it ready; an in-place update of the table makes a new buffer."""
+    from turbot5_amd import ops
+    B, H, M, D = 2, 5, 700, 64
+    q, k, v = (rnd(B, H, M, D, seed=90 + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+    table = rnd(32, H, seed=93, scale=1.0).to(gpu_device)
+    run = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0).cpu()  # noqa: E731
+    ops._BIAS_LUTS.clear()
+    ops.BIAS_LUT_CACHE = False
+    try:
+        plain = run()
+    finally:
+        ops.BIAS_LUT_CACHE = True
+    assert len(ops._BIAS_LUTS) == 0
+    first, second = run(), run()
+    assert len(ops._BIAS_LUTS) == 1
+    assert torch.equal(plain.view(torch.int16), first.view(torch.int16))
+    assert torch.equal(plain.view(torch.int16), second.view(torch.int16))
+    table.mul_(-0.5)   # same storage, new values
+    third = run()
+    assert len(ops._BIAS_LUTS) == 2
+    want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), table.cpu(), causal, 1.0)
+    assert (third.float() - want).abs().max().item() <= TOL[torch.bfloat16]
+    assert not torch.equal(third.view(torch.int16), plain.view(torch.int16))
+
+
+@pytest.mark.parametrize("tdtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("layout", ["plain", "offset", "transposed"])
+def test_bias_table_dtypes_and_layouts(gpu_device, tdtype, layout):
+    """The kernel reads the (NUM_BUCKETS, H) table in its own type and strides: 16-bit tables, a table that
+    starts in the middle of a 4-byte word, and the transposed (H, NUM_BUCKETS) storage, with and without
+    the LUT buffer."""
+    from turbot5_amd import ops
+    B, H, M, D = 1, 3, 300, 64
+    q, k, v = (rnd(B, H, M, D, seed=100 + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+    vals = rnd(32, H, seed=103, scale=1.0).to(tdtype)
+    if layout == "plain":
+        table = vals.to(gpu_device)
+    elif layout == "offset":
+        buf = torch.zeros(32 * H + 1, dtype=tdtype, device=gpu_device)
+        buf[1:] = vals.reshape(-1).to(gpu_device)
+        table = buf[1:].view(32, H)
+    else:
+        table = vals.t().contiguous().to(gpu_device).t()
+    assert table.shape == (32, H)
+    want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), vals.float(), False, 1.0)
+    for cache in (False, True):
+        ops.BIAS_LUT_CACHE = cache
+        try:
+            got = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0)
+        finally:
+            ops.BIAS_LUT_CACHE = True
+        assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16], (cache, layout, tdtype)

@@ -32,7 +32,7 @@ def test_header_symbols_are_exported(lib):
 
 def test_struct_sizes_follow_the_header(lib):
     # natural alignment, no packing: catches a field added on one side only
-    assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8
+    assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 8 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias)

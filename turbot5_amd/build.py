@@ -24,6 +24,7 @@ UNITS = [
     ("splitk.o", "splitk.hip", []),
     ("rmsnorm.o", "rmsnorm.hip", []),
     ("plan.o", "plan.hip", []),
+    ("lut.o", "lut.hip", []),
     ("attn_fwd_bf16.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=0"]),
     ("attn_fwd_f32.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=1"]),
     ("attn_fwd_f16.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=2"]),
@@ -48,7 +49,7 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
-def build(verbose: bool = False, jobs: int = 7, extra_flags=()) -> str:
+def build(verbose: bool = False, jobs: int = 8, extra_flags=()) -> str:
     """Compile every translation unit and link the shared library; returns its path."""
     os.makedirs(OBJ, exist_ok=True)
     hipcc = _hipcc()

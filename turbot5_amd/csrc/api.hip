@@ -138,6 +138,23 @@ static int fill_bias(const t5a_bias& b, bool bidirectional, FwdParams* p) {
     return make_bucket_spec(bidirectional, b.num_buckets, b.max_distance, &p->bs);
 }
 
+// Optional buffer with the distance LUTs of all heads: checked, built on the first use, handed to the kernel.
+static int prepare_lut(const t5a_bias& b, bool causal, hipStream_t stream, FwdParams* p) {
+    if (b.table == nullptr || b.lut == nullptr) return T5A_OK;
+    const int64_t need = bias_lut_bytes(p->H, p->bs, causal);
+    if (need == 0) return T5A_OK;   // not usable for these parameters: the kernel builds its LUTs itself
+    if (b.lut_bytes < need)
+        return fail(T5A_ERR_WORKSPACE, "bias.lut too small: %lld bytes, t5a_bias_lut_bytes() asks for %lld",
+                    (long long)b.lut_bytes, (long long)need);
+    if ((reinterpret_cast<uintptr_t>(b.lut) & 15) != 0) return fail(T5A_ERR_STRIDE, "bias.lut must be 16-byte aligned");
+    if (b.lut_ready == 0) {
+        hipError_t e = launch_bias_lut(*p, causal, static_cast<float*>(b.lut), stream);
+        if (e != hipSuccess) return fail(T5A_ERR_LAUNCH, "bias LUT build: %s", hipGetErrorString(e));
+    }
+    p->lut_global = static_cast<const float*>(b.lut);
+    return T5A_OK;
+}
+
 static int finish(hipError_t e, const char* what) {
     if (e != hipSuccess) return fail(T5A_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
     return T5A_OK;
@@ -162,6 +179,12 @@ extern "C" {
 int t5a_version(void) { return 100; }
 
 const char* t5a_last_error(void) { return g_err; }
+
+int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t causal) {
+    BucketSpec bs;
+    if (H <= 0 || make_bucket_spec(causal == 0, num_buckets, max_distance, &bs) != T5A_OK) return 0;
+    return bias_lut_bytes(H, bs, causal != 0);
+}
 
 int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t* out) {
     if (out == nullptr) return fail(T5A_ERR_NULL, "out is NULL");
@@ -233,6 +256,7 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     if (a->causal != 0 && p.tiles_per_seq > 1) causal_slices(&p, a->dtype, a->D);
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
+    if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
 }
 
@@ -283,6 +307,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     p.align_end = 1;
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
+    if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     const int64_t need = t5a_varlen_workspace_bytes(a->B, a->H, a->total_q);
     if (a->workspace != nullptr && need > 0) {
         // launch plan: per-XCD item lists of equal work, longest first, built on the device
@@ -378,6 +403,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;
     hipStream_t s = (hipStream_t)stream;
+    if ((rc = prepare_lut(a->bias, false, s, &p))) return rc;
 
     if (a->pattern == T5A_PATTERN_BLOCK) {
         if (a->L < a->block_len) {

@@ -49,6 +49,7 @@
 #include <type_traits>
 
 #include "t5a_internal.h"
+#include "lut_device.h"
 
 namespace t5a {
 
@@ -108,46 +109,12 @@ constexpr int BM = 128;      // query rows per workgroup
 // tiles keep two workgroups per compute unit
 template <typename T, int D> constexpr int tile_keys() { return sizeof(T) == 2 && D == 128 ? 32 : 64; }
 constexpr int NTHREADS = 256;
-// The distance LUT extends this far past the saturation distance on both sides.  A tile that takes
-// the LUT path has at least one unsaturated (row, key) pair, and a wavefront tile spans 32 rows x
-// 64 keys, so none of its distances lies more than 94 past saturation: lookups need no clamping.
-constexpr int LUT_PAD = 96;
 constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
 #ifndef OCC
 #define OCC 2
 #endif
 
-__device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {
-    int out = 0, d;
-    if (s.bidirectional) { out = rel > 0 ? s.nb : 0; d = rel < 0 ? -rel : rel; }
-    else { d = rel < 0 ? -rel : 0; }
-    if (d < s.max_exact) return out + d;
-    // the first 16 thresholds come in with one scalar load and are compared without a loop
-    // (unused slots hold INT_MAX); the loop only runs for unusually fine bucketings
-    int b = s.max_exact;
-#pragma unroll
-    for (int t = 0; t < 16; ++t) b += (d >= s.thr[t]) ? 1 : 0;
-    for (int t = 16; t < s.n_thr; ++t) b += (d >= s.thr[t]) ? 1 : 0;
-    return out + b;
-}
-
-__device__ __forceinline__ float load_table(const void* table, int dtype, int64_t off) {
-    if (dtype == T5A_F32) return reinterpret_cast<const float*>(table)[off];
-    if (dtype == T5A_BF16) return static_cast<float>(reinterpret_cast<const __bf16*>(table)[off]);
-    return static_cast<float>(reinterpret_cast<const _Float16*>(table)[off]);
-}
-
-// Table element fetched from inline assembly, so that the kernel decides how long to wait for it
-// (see the prologue): `raw` receives the element's bits, zero-extended for the 16-bit types.
-__device__ __forceinline__ void load_table_async(const void* table, int dtype, int64_t off, unsigned& raw) {
-    if (dtype == T5A_F32) {
-        const float* a = reinterpret_cast<const float*>(table) + off;
-        asm volatile("global_load_dword %0, %1, off" : "+v"(raw) : "v"(a) : "memory");
-    } else {
-        const unsigned short* a = reinterpret_cast<const unsigned short*>(table) + off;
-        asm volatile("global_load_ushort %0, %1, off" : "+v"(raw) : "v"(a) : "memory");
-    }
-}
+// table element from its bits (zero-extended for the 16-bit types)
 __device__ __forceinline__ float table_value(unsigned raw, int dtype) {
     if (dtype == T5A_F32) return __uint_as_float(raw);
     if (dtype == T5A_BF16) return __uint_as_float(raw << 16);
@@ -190,6 +157,14 @@ __device__ __forceinline__ void lds_dma_16(u32x4 rs, unsigned lds_addr, int voff
     const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
                         (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+}
+
+// one dword per lane: 256 consecutive bytes of LDS
+__device__ __forceinline__ void lds_dma_4(u32x4 rs, unsigned lds_addr, int voffset) {
+    const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
+                        (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
                  :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
 }
 
@@ -260,12 +235,6 @@ struct Geometry {
     // (rows of 256 bytes span all banks: there the four keys of a read go to four different quarters)
     static __device__ __forceinline__ int vrow_swz(int key) { return D == 128 ? (key & 3) << 2 : ((key >> 1) & 1) << 2; }
 };
-
-// floats per shifted copy of the distance LUT (host and device agree through this)
-__host__ __device__ inline int lut_quads(int sat, bool causal) {
-    const int entries = sat + LUT_PAD + (causal ? 0 : sat) + LUT_PAD + 1;   // rel = -sat-PAD .. (sat|0)+PAD
-    return (entries + 3 + 3) / 4 + 1;                                      // + 3 for the shifted copies
-}
 
 template <typename T, int D, int MODE, bool CAUSAL>
 __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) void fwd_kernel(const FwdParams p) {
@@ -564,15 +533,44 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     const float log2e = 1.4426950408889634f;
     // The head's table column: with at most 64 buckets, lane b of every wavefront fetches bucket b up
     // front and the LUT entries pick their value with a lane permute; larger tables are read per entry.
-    // Order of the prologue's memory requests: Q rows, table column, then the first K/V tiles.  Loads
-    // complete in order, so "at most the tile requests outstanding" means Q and the column are here,
-    // and the LUT is built while the tiles are still in flight (built after a wait for everything,
-    // it made up half of the 5 us a work item spends outside its tile loop).
+    // A caller-provided buffer may instead hold the LUTs of all heads, built once per table (lut.hip): the
+    // head's image (4 * qlen floats) is then fetched as it is.
+    //
+    // LDS-DMA geometries fetch either of them with LDS-DMA requests of their own, issued BEFORE the first
+    // K/V tiles: requests complete in order, so "at most the tile requests outstanding" means the column
+    // (or this wavefront's pieces of the image) has landed, and the LUT is built while the tiles are still
+    // in flight.  Nothing of this passes through vector registers: the compiler does not know that a
+    // register written by a load issued from inline assembly is still in flight and may copy it too early.
     const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
     const bool col_in_lanes = nbt <= 64;
-    unsigned tcol_raw = 0;
-    if (has_bias && col_in_lanes && lane < nbt)
-        load_table_async(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead, tcol_raw);
+    const bool lut_cached = has_bias && p.lut_global != nullptr;   // the host checked qlen <= 512
+    const int col_esize = p.table_dtype == T5A_F32 ? 4 : 2;
+    // byte offset of this lane's bucket in the table, from the 4-byte aligned address at or below its start
+    const unsigned col_misalign = (unsigned)(reinterpret_cast<uintptr_t>(p.table) & 3);
+    const unsigned col_byte = col_misalign +
+        (unsigned)(((int64_t)(lane < nbt ? lane : 0) * p.t_sbucket + (int64_t)h * p.t_shead) * col_esize);
+    const int lut_region = (4 * qlen + 255) & ~255;   // floats: the image, rounded up to whole 1 KB requests
+    float* col_stage = lut + lut_region + wave * 64;  // 64 dwords per wavefront behind it
+    float tcol = 0.f;
+    if constexpr (DMA) {
+        if (lut_cached) {
+            const u32x4 rs = make_rsrc_words(p.lut_global + (size_t)h * (4 * qlen), (unsigned)(qlen * 16));
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int first = c * NTHREADS + wave * 64;   // first 16-byte piece of this request
+                if (first < qlen)   // pieces past the image read as zeros into the slack behind it
+                    lds_dma_16(rs, lds_base + (unsigned)(NSV * V_TILE + NSK * K_TILE) * ES + first * 16, (first + lane) * 16);
+            }
+        } else if (has_bias && col_in_lanes) {
+            const unsigned col_bytes = col_misalign +
+                (unsigned)(((int64_t)(nbt - 1) * p.t_sbucket + (int64_t)(p.H - 1) * p.t_shead + 1) * col_esize);
+            const u32x4 rs = make_rsrc_words(reinterpret_cast<const char*>(p.table) - col_misalign, (col_bytes + 3) & ~3u);
+            lds_dma_4(rs, lds_base + (unsigned)(NSV * V_TILE + NSK * K_TILE) * ES + (lut_region + wave * 64) * 4,
+                      (int)(col_byte & ~3u));
+        }
+    } else if (has_bias && col_in_lanes && lane < nbt && !lut_cached) {
+        tcol = load_table(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
+    }
     // request the first tiles: they arrive while the bias LUT is built
     if constexpr (DMA) {
         if constexpr (DENSE) {
@@ -583,32 +581,22 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             for (int i = 0; i < 4; ++i) dma_tile(i, false);
             for (int i = 0; i < 3; ++i) dma_tile(i, true);
         }
-    }
-
-    constexpr int PROLOGUE_TILE_REQUESTS = DMA ? 7 * G::SPW : 0;   // per wavefront, all issued after the column load
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(tcol_raw) : "n"(PROLOGUE_TILE_REQUESTS));
-    if (has_lut) {
-        const float tcol = table_value(tcol_raw, p.table_dtype) * log2e;
-        // one evaluation per distance; the value goes to all four shifted copies:
-        // copy a, slot i holds the distance i + a - padl
-        for (int e0 = 0; e0 < qlen + 3; e0 += NTHREADS) {   // uniform trip count: the permute needs every lane
-            const int e = e0 + tid;
-            const int rel = e - padl;
-            float val = 0.f;
-            if (has_bias) {
-                const int bk = bucket_of(p.bs, rel);
-                if (col_in_lanes)
-                    val = __int_as_float(__builtin_amdgcn_ds_bpermute(bk << 2, __float_as_int(tcol)));
-                else
-                    val = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
-            }
-            if (CAUSAL && rel > 0) val = -INFINITY;
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                const int i = e - a;
-                if (i >= 0 && i < qlen && e < qlen + 3) lut[a * qlen + i] = val;
-            }
+        // everything older than the tile requests; the clobber keeps the LDS read below behind the wait
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(7 * G::SPW) : "memory");
+        if (!lut_cached && has_bias && col_in_lanes) {
+            const unsigned raw = __float_as_uint(col_stage[lane]);
+            const unsigned el = col_esize == 4 ? raw : ((raw >> (8 * (col_byte & 2))) & 0xffffu);
+            tcol = table_value(el, p.table_dtype) * log2e;
         }
+    }
+    if (lut_cached) {
+        if constexpr (!DMA) {
+            const f32x4* src = reinterpret_cast<const f32x4*>(p.lut_global + (size_t)h * (4 * qlen));
+            for (int idx = tid; idx < qlen; idx += NTHREADS) reinterpret_cast<f32x4*>(lut)[idx] = src[idx];
+        }
+    } else if (has_lut) {
+        lut_fill<CAUSAL>(lut, p.bs, p.table, p.table_dtype, p.t_sbucket, p.t_shead, h, has_bias, tcol, col_in_lanes,
+                         padl, qlen, tid, NTHREADS);
     }
     if (D < 32) {  // the part of V past head_dim feeds the MFMA: keep it zero
         for (int idx = tid; idx < NSV * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
@@ -1175,7 +1163,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
 template <typename T, int D, int MODE, bool CAUSAL>
 static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
     const int sat = p.table != nullptr ? p.bs.sat : 0;
-    const size_t lut_bytes = (size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float);
+    // the LUT image rounded up to 1 KB (its LDS-DMA requests are that long) and 256 bytes per wavefront
+    // for the table column
+    const size_t lut_bytes = (((size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float) + 1023) & ~(size_t)1023) + 1024;
     const size_t smem = Geometry<T, D>::kTileBytes + lut_bytes;
     auto kern = fwd_kernel<T, D, MODE, CAUSAL>;
     static std::atomic<size_t> granted{0};   // per instantiation: largest dynamic LDS size already allowed

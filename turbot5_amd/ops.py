@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+from collections import OrderedDict
 from typing import Optional, Tuple
 
 import torch
@@ -48,7 +49,39 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
     return t if ok else t.contiguous()
 
 
-def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_distance: int, ref: torch.Tensor):
+# Distance LUTs of the bias tables seen lately, built on the device by the first launch that uses a table and
+# fetched by the later ones.  Keyed by the table's identity and version (so an optimiser step or any other
+# in-place update makes a new entry), the bucket parameters and the stream the build was queued on; the entry
+# keeps the table alive, so its address cannot be taken by another tensor.
+_BIAS_LUTS: "OrderedDict[tuple, tuple]" = OrderedDict()
+BIAS_LUT_CACHE = True
+
+
+def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int, causal: bool, ref: torch.Tensor):
+    stream = _stream(ref)
+    if not BIAS_LUT_CACHE or torch.cuda.is_current_stream_capturing():
+        return None   # a build recorded into a graph would not have run when the next eager launch reads it
+    key = (bias.data_ptr(), bias._version, tuple(bias.shape), bias.stride(), bias.dtype, num_buckets, max_distance,
+           bool(causal), str(ref.device), stream)
+    hit = _BIAS_LUTS.get(key)
+    if hit is None:
+        nbytes = L.load().t5a_bias_lut_bytes(H, num_buckets, max_distance, int(bool(causal)))
+        if nbytes <= 0:
+            return None
+        lut = torch.empty(nbytes, device=ref.device, dtype=torch.uint8)
+        _BIAS_LUTS[key] = (bias, lut)
+        while len(_BIAS_LUTS) > 64:
+            _BIAS_LUTS.popitem(last=False)
+        b.lut_ready = 0
+    else:
+        lut = hit[1]
+        b.lut_ready = 1
+    b.lut, b.lut_bytes = lut.data_ptr(), lut.numel()
+    return lut
+
+
+def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_distance: int, ref: torch.Tensor,
+                 causal: bool = False):
     b = L.T5ABias()
     if bias is None:
         b.table = None
@@ -66,7 +99,8 @@ def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_dis
     b.max_distance = max_distance
     b.stride_bucket = table.stride(0)
     b.stride_head = table.stride(1)
-    return b, table   # keep `table` alive until the launch has been queued
+    lut = _bias_lut(b, bias, H, num_buckets, max_distance, causal, ref) if table.data_ptr() == bias.data_ptr() else None
+    return b, (table, lut)   # keep both alive until the launch has been queued
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -125,7 +159,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q_), _strides3(k_), _strides3(v_), _strides3(o)
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
-    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, causal)
     with _on_device(q):
         L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
     return (o, lse) if return_lse else o
@@ -217,7 +251,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     a.total_q, a.total_k = total_q, total_k
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
-    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, causal)
     lib = L.load()
     # building a plan costs about 15 us: worth it from a few thousand items on, earlier when shared
     items = (total_q // 128 + B) * H
