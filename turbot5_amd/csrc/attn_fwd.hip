@@ -157,7 +157,7 @@ __device__ __forceinline__ void lds_dma_16(u32x4 rs, unsigned lds_addr, int voff
     const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
                         (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
 }
 
 // one dword per lane: 256 consecutive bytes of LDS
@@ -165,7 +165,7 @@ __device__ __forceinline__ void lds_dma_4(u32x4 rs, unsigned lds_addr, int voffs
     const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
                         (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
 }
 
 // Two requests that share one descriptor and one LDS base: the second carries an instruction offset of
@@ -176,7 +176,7 @@ __device__ __forceinline__ void lds_dma_16x2(unsigned lo, unsigned hi, unsigned 
                         (unsigned)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
                  "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory", "m0");
 }
 
 // s_waitcnt vmcnt(N) alone (six-bit count: bits 3:0 and 15:14), the other counters left open
