@@ -239,6 +239,7 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
         if ((rc = check_rows("k", a->N, a->k_strides[2], a->dtype))) return rc;
         if ((rc = check_rows("v", a->N, a->v_strides[2], a->dtype))) return rc;
     }
+    if ((rc = check_rows("q", a->M, a->q_strides[2], a->dtype))) return rc;
     FwdParams p;
     memset(&p, 0, sizeof(p));
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
@@ -288,6 +289,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
         if ((rc = check_rows("k", a->max_seqlen_k, a->k_strides[0], a->dtype))) return rc;
         if ((rc = check_rows("v", a->max_seqlen_k, a->v_strides[0], a->dtype))) return rc;
     }
+    if ((rc = check_rows("q", a->max_seqlen_q, a->q_strides[0], a->dtype))) return rc;
     FwdParams p;
     memset(&p, 0, sizeof(p));
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
@@ -380,6 +382,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
     if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
     if ((rc = check_tensor("o", a->o, a->o_strides, 3, unit))) return rc;
+    if ((rc = check_rows("q", a->L, a->q_strides[2], a->dtype))) return rc;
     if ((rc = check_rows("k", a->L, a->k_strides[2], a->dtype))) return rc;
     if ((rc = check_rows("v", a->L, a->v_strides[2], a->dtype))) return rc;
     if (a->pattern == T5A_PATTERN_TGLOBAL && a->n_side > 0) {

@@ -249,6 +249,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     constexpr int ES = sizeof(T);
     constexpr int BN = G::BN, NT = G::NT;
     constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
+    // head_dim 64, 16-bit types: the Q rows are staged through LDS by LDS-DMA as well (see the prologue)
+    constexpr bool QDMA = G::DMA && D == 64;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr bool DMA = G::DMA;
@@ -514,7 +516,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             qraw[c] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (row_ok) qraw[c] = *reinterpret_cast<const f32x4*>(qp + (int64_t)irow * p.q_sr + 4 * c);
         }
-    } else {
+    } else if constexpr (!QDMA) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
 #pragma unroll
@@ -552,6 +554,23 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     const int lut_region = (4 * qlen + 255) & ~255;   // floats: the image, rounded up to whole 1 KB requests
     float* col_stage = lut + lut_region + wave * 64;  // 64 dwords per wavefront behind it
     float tcol = 0.f;
+    // With QDMA the order of the prologue's requests is  K0 V0 | Q rows | column or LUT image | K1 V1 K2 V2,
+    // and K3 follows once every wavefront has taken its Q rows out of LDS: the rows are staged in the last
+    // stage of the K ring (wavefronts 0, 1) and of the V ring (2, 3), 4 KB each, which the loop fills first
+    // with K3 and V3.  Requests complete in order, so "at most K1 V1 K2 V2 outstanding" means that K0, V0,
+    // Q and the column have landed: the LUT is built and the first product formed while the rest is in
+    // flight.  (Q loaded into registers by the compiler would be waited for with "nothing outstanding".)
+    const unsigned q_stage = wave < 2 ? (unsigned)(NSV * V_TILE + 3 * K_TILE) * ES + wave * 4096u
+                                      : (unsigned)(3 * V_TILE) * ES + (wave - 2) * 4096u;
+    if constexpr (QDMA) {
+        if constexpr (DENSE) { cursor_seek(0, 0); cursor_dma(0, 0); }
+        else { dma_tile(0, false); dma_tile(0, true); }
+        const int q_row_bytes = (int)p.q_sr * ES;
+        const u32x4 rs = make_rsrc_words(qp, row_end > 0 ? (unsigned)(row_end - 1) * (unsigned)q_row_bytes + D * ES : 0u);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)   // 8 rows of 128 bytes per request; rows past the end arrive as zeros
+            lds_dma_16(rs, lds_base + q_stage + r * 1024, (iw0 + 8 * r + (lane >> 3)) * q_row_bytes + (lane & 7) * 16);
+    }
     if constexpr (DMA) {
         if (lut_cached) {
             const u32x4 rs = make_rsrc_words(p.lut_global + (size_t)h * (4 * qlen), (unsigned)(qlen * 16));
@@ -573,7 +592,10 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     }
     // request the first tiles: they arrive while the bias LUT is built
     if constexpr (DMA) {
-        if constexpr (DENSE) {
+        if constexpr (QDMA) {
+            if constexpr (DENSE) { cursor_dma(1, 1); cursor_dma(2, 2); }   // K1 V1, K2 V2
+            else { dma_tile(1, false); dma_tile(1, true); dma_tile(2, false); dma_tile(2, true); }
+        } else if constexpr (DENSE) {
             cursor_seek(0, 0);
             cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
             dma_tile(3, false);                                     // K3
@@ -581,8 +603,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             for (int i = 0; i < 4; ++i) dma_tile(i, false);
             for (int i = 0; i < 3; ++i) dma_tile(i, true);
         }
-        // everything older than the tile requests; the clobber keeps the LDS read below behind the wait
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(7 * G::SPW) : "memory");
+        // everything older than these tile requests; the clobber keeps the LDS reads below behind the wait
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"((QDMA ? 4 : 7) * G::SPW) : "memory");
         if (!lut_cached && has_bias && col_in_lanes) {
             const unsigned raw = __float_as_uint(col_stage[lane]);
             const unsigned el = col_esize == 4 ? raw : ((raw >> (8 * (col_byte & 2))) & 0xffffu);
@@ -606,6 +628,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     const float c_pos = has_bias ? lut[qlen - 1] : 0.f;          // every key far after it (non-causal)
 
     // ---------------------------------------------------------------- Q fragments: pre-scale by sm_scale*log2(e)
+    if constexpr (QDMA) {
+        const T* qs_rows = reinterpret_cast<const T*>(smem + q_stage);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v8*>(qs_rows + lr * D + (2 * s + hh) * 8);
+    }
     if constexpr (F32) {
 #pragma unroll
         for (int c = 0; c < D / 4; ++c) {
@@ -1010,21 +1037,27 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // have landed.
     f32x16 sta[NT], stb[NT];
     TileClass tc = classify(0);
-    if constexpr (DMA) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the tiles requested at the top have landed
-    } else if (ntiles > 0) {
-        load_tile_k(0); load_tile_v(0);
-        store_tile_k(0); store_tile_v(0);
-        if (ntiles > 1) { load_tile_k(1); store_tile_k(1); }
+    if constexpr (QDMA) {
+        // K0 and V0 landed before the barrier that published the LUT
+    } else {
+        if constexpr (DMA) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the tiles requested at the top have landed
+        } else if (ntiles > 0) {
+            load_tile_k(0); load_tile_v(0);
+            store_tile_k(0); store_tile_v(0);
+            if (ntiles > 1) { load_tile_k(1); store_tile_k(1); }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (tc.side != 0) refill_cm(tc.side);
     if (ntiles > 0 && !tc.skip) {
         v8 ka0[NT][KS];
         read_k(0, ka0);
         compute_s(tc, 0, ka0, sta);
     }
+    if constexpr (QDMA) wait_vmcnt<3 * G::SPW>();   // K1 has landed; V1 K2 V2 may still be in flight
     __syncthreads();   // the first step overwrites the K buffer this product was read from
+    if constexpr (QDMA) dma_tile(3, false);         // K3, into the stage that held the Q rows of two wavefronts
 
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         const int kbuf_next = DMA ? (t + 1) % NSK : (t + 1) & 1;
