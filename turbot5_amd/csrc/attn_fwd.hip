@@ -35,7 +35,8 @@
 //
 // The T5 relative-position bias is not materialised.  Each workgroup expands
 // its head's column of the (num_buckets, H) table into a distance-indexed LUT
-// in LDS covering the distances at which buckets still change; for causal
+// in LDS covering the distances at which buckets still change (or fetches the
+// finished image from a per-table buffer, lut.hip); for causal
 // attention the LUT holds -inf for every future key, so the diagonal needs no
 // separate mask.  Four copies of the LUT, shifted by 0..3 entries, let a lane
 // fetch the biases of four consecutive keys with one aligned 16-byte read,
