@@ -58,11 +58,10 @@ BIAS_LUT_CACHE = True
 
 
 def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int, causal: bool, ref: torch.Tensor):
-    stream = _stream(ref)
     if not BIAS_LUT_CACHE or torch.cuda.is_current_stream_capturing():
         return None   # a build recorded into a graph would not have run when the next eager launch reads it
-    key = (bias.data_ptr(), bias._version, tuple(bias.shape), bias.stride(), bias.dtype, num_buckets, max_distance,
-           bool(causal), str(ref.device), stream)
+    key = (bias.data_ptr(), bias._version, bias.stride(0), bias.stride(1), bias.dtype, H, num_buckets, max_distance,
+           bool(causal), ref.device.index, _stream(ref))
     hit = _BIAS_LUTS.get(key)
     if hit is None:
         nbytes = L.load().t5a_bias_lut_bytes(H, num_buckets, max_distance, int(bool(causal)))
