@@ -79,6 +79,9 @@ typedef struct t5a_bias {
  * the unidirectional buckets, as in t5a_fwd_dense. */
 int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t causal);
 
+/* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
+ * it passes a struct (a stale library would read pointers from the wrong offsets). */
+#define T5A_ABI_VERSION 103
 int t5a_version(void);
 const char* t5a_last_error(void);
 

@@ -27,7 +27,7 @@ def test_header_symbols_are_exported(lib):
     handle = lib.load()
     for name in declared:
         assert getattr(handle, name) is not None
-    assert handle.t5a_version() >= 100
+    assert handle.t5a_version() == lib.ABI_VERSION == int(re.search(r"#define T5A_ABI_VERSION (\d+)", header).group(1))
 
 
 def test_struct_sizes_follow_the_header(lib):

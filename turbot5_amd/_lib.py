@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
+ABI_VERSION = 103   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
@@ -104,6 +105,9 @@ def load() -> C.CDLL:
                 "there is no fallback path")
         lib = C.CDLL(LIB_PATH)
         lib.t5a_version.restype = C.c_int
+        if lib.t5a_version() != ABI_VERSION:   # the structs below would not match what the library reads
+            raise ImportError(f"{LIB_PATH} has ABI version {lib.t5a_version()}, this binding expects {ABI_VERSION}: "
+                              "rebuild it (`python -m turbot5_amd.build`)")
         lib.t5a_last_error.restype = C.c_char_p
         lib.t5a_bucket_lut.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32)]
         lib.t5a_bucket_lut.restype = C.c_int

@@ -176,7 +176,7 @@ using namespace t5a;
 
 extern "C" {
 
-int t5a_version(void) { return 100; }
+int t5a_version(void) { return T5A_ABI_VERSION; }
 
 const char* t5a_last_error(void) { return g_err; }
 
