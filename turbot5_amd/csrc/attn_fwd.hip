@@ -385,6 +385,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     //   0: i + P     1: i % block_len + G (block pattern, global keys)     2: i / aux (side tokens)
     const T* seg_k[2]; const T* seg_v[2];
     int seg_ksr[2], seg_vsr[2];      // row strides in bytes
+    // (read with explicit selects, never with a run-time index: an indexed private array lives in scratch
+    // memory, and a scratch load waits for every tile request in flight)
     int seg_start[2], seg_end[2], seg_lend[2], seg_kind[2], seg_win[2];
     int nseg = 1;
     seg_k[0] = reinterpret_cast<const T*>(p.k) + k_off;
@@ -436,7 +438,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
 
     auto tile_of = [&](int t, int& sg, int& j0) {
         sg = t >= seg_nt[0] ? 1 : 0;
-        j0 = seg_start[sg] + (t - (sg ? seg_nt[0] : 0)) * BN;
+        j0 = (sg ? seg_start[1] : seg_start[0]) + (t - (sg ? seg_nt[0] : 0)) * BN;
     };
     // LDS-DMA staging: a wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses
     // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
@@ -446,7 +448,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         if constexpr (DMA) {
             int sg, j0; tile_of(t, sg, j0);
             const u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
-            const int sr = is_v ? seg_vsr[sg] : seg_ksr[sg];
+            const int sr = is_v ? (sg ? seg_vsr[1] : seg_vsr[0]) : (sg ? seg_ksr[1] : seg_ksr[0]);
             if (stage < 0) stage = is_v ? t % NSV : t % NSK;
             const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
 #pragma unroll
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     auto load_tile_k = [&](int t) {
         int sg, j0; tile_of(t, sg, j0);
         const __amdgpu_buffer_rsrc_t krs = sg ? seg_krs[1] : seg_krs[0];
-        const int ksr = seg_ksr[sg];
+        const int ksr = (sg ? seg_ksr[1] : seg_ksr[0]);
         // the whole byte offset goes into the vector operand: only that one is range checked
 #pragma unroll
         for (int c = 0; c < K_PER_T; ++c) {
@@ -679,7 +681,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     auto load_tile_v = [&](int t) {
         int sg, j0; tile_of(t, sg, j0);
         const __amdgpu_buffer_rsrc_t vrs = sg ? seg_vrs[1] : seg_vrs[0];
-        const int vsr = seg_vsr[sg];
+        const int vsr = (sg ? seg_vsr[1] : seg_vsr[0]);
         if constexpr (F32) {
 #pragma unroll
             for (int c = 0; c < V_PER_T; ++c) {
@@ -787,8 +789,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             return c;
         }
         tile_of(t, c.sg, c.j0);
-        const int kind = seg_kind[c.sg];
-        const bool win = seg_win[c.sg] != 0;
+        const int kind = (c.sg ? seg_kind[1] : seg_kind[0]);
+        const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
         int qlo, qhi;
         if (kind == 0) { qlo = iw0 + P; qhi = iw1 + P; }
         else if (kind == 1) { qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
@@ -800,7 +802,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         const bool left_sat = rel_max <= -sat && (!CAUSAL || rel_max <= 0);
         const bool right_sat = !CAUSAL && rel_min >= sat;
         c.use_lut = has_lut && !(left_sat || right_sat);
-        c.need_mask = c.j0 + BN > seg_end[c.sg];
+        c.need_mask = c.j0 + BN > (c.sg ? seg_end[1] : seg_end[0]);
         if (win) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
         c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
         return c;
@@ -826,7 +828,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     for (int r = 0; r < 16; ++r) cm[r] = 0.f;
 
     auto lane_qpos = [&](int sg) {   // this lane's query position in the segment's bias geometry
-        const int kind = seg_kind[sg];
+        const int kind = (sg ? seg_kind[1] : seg_kind[0]);
         const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
         if (kind == 0) return ir + P;
         if (kind == 1) return ir % p.block_len + p.aux;
@@ -897,8 +899,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // mask, row max, lazy raise of the running max; returns true when m_run changed
     auto softmax_head = [&](const TileClass& c, f32x16 (&st)[NT]) {
         if (c.need_mask) {   // keys past the end of the segment, or outside the window
-            const int s_end = seg_end[c.sg];
-            const bool win = seg_win[c.sg] != 0;
+            const int s_end = (c.sg ? seg_end[1] : seg_end[0]);
+            const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
             const int qpos = lane_qpos(c.sg);
             const int jl = c.j0 + 4 * hh;
 #pragma unroll
