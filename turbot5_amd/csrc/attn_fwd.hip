@@ -902,15 +902,17 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             const int s_end = (c.sg ? seg_end[1] : seg_end[0]);
             const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
             const int qpos = lane_qpos(c.sg);
-            const int jl = c.j0 + 4 * hh;
+            // this lane's row sees the keys [lo, hi): one subtraction and one unsigned compare per element
+            const int lo = win ? max(0, qpos - p.block_len + 1) : 0;
+            const int hi = win ? min(s_end, qpos + p.block_len) : s_end;
+            const unsigned span = (unsigned)max(hi - lo, 0);
+            const int jl = c.j0 + 4 * hh - lo;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int j = jl + 32 * nt + 8 * (r >> 2) + (r & 3);
-                    bool ok = j < s_end;
-                    if (win) { const int rel = j - qpos; ok = ok && rel < p.block_len && rel > -p.block_len; }
-                    st[nt][r] = ok ? st[nt][r] : -INFINITY;
+                    const unsigned j = (unsigned)(jl + 32 * nt + 8 * (r >> 2) + (r & 3));
+                    st[nt][r] = j < span ? st[nt][r] : -INFINITY;
                 }
         }
         // st already holds (score - m_run)
