@@ -185,26 +185,52 @@ __global__ __launch_bounds__(SK_THREADS) void splitk_partial_kernel(const SplitK
     }
 }
 
+// Merge over splits, one wavefront per output row.  The splits' log-sum-exps and weights are read with one
+// lane per split (not one after the other), the weights go through LDS, and the weighted sum over the splits
+// runs four splits at a time so that their loads are in flight together: with 40 and more splits the serial
+// version spent its time waiting for one load after the other.
 template <typename T, int D>
-__global__ __launch_bounds__(D < 64 ? 64 : D) void splitk_merge_kernel(const SplitKParams p) {
+__global__ __launch_bounds__(64) void splitk_merge_kernel(const SplitKParams p) {
+    constexpr int MAXS = 256;            // weights kept in LDS; more splits fall back to recomputing them
+    __shared__ float s_w[MAXS];
     const int m = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int d = threadIdx.x;
-    if (d >= D) return;
+    const int lane = threadIdx.x;
     const int64_t base = (((int64_t)b * p.H + h) * p.S) * p.M + m;   // + s * M
     float gm = -INFINITY;
-    for (int s = 0; s < p.S; ++s) gm = fmaxf(gm, p.part_m[base + (int64_t)s * p.M]);
-    float wsum = 0.f, val = 0.f;
-    for (int s = 0; s < p.S; ++s) {
+    for (int s = lane; s < p.S; s += 64) gm = fmaxf(gm, p.part_m[base + (int64_t)s * p.M]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) gm = fmaxf(gm, __shfl_xor(gm, o, 64));
+    auto weight = [&](int s) {
         const int64_t row = base + (int64_t)s * p.M;
         const float l = p.part_l[row];
-        if (l > 0.f) {
-            const float wgt = l * __expf(p.part_m[row] - gm);
-            wsum += wgt;
-            val = fmaf(p.part_o[row * D + d], wgt, val);
-        }
+        return l > 0.f ? l * __expf(p.part_m[row] - gm) : 0.f;
+    };
+    float wsum = 0.f;
+    for (int s = lane; s < p.S; s += 64) {
+        const float w = weight(s);
+        if (s < MAXS) s_w[s] = w;
+        wsum += w;
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) wsum += __shfl_xor(wsum, o, 64);
+    __syncthreads();
     T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)m * p.o_sr;
-    op[d] = SkLoad<T>::cvt(wsum > 0.f ? val / wsum : 0.f);
+    for (int d = lane; d < D; d += 64) {
+        float val = 0.f;
+        int s = 0;
+        for (; s + 4 <= p.S && s + 4 <= MAXS; s += 4) {
+            float x[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[i] = p.part_o[(base + (int64_t)(s + i) * p.M) * D + d];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) val = s_w[s + i] > 0.f ? fmaf(x[i], s_w[s + i], val) : val;   // an empty split's row may hold anything
+        }
+        for (; s < p.S; ++s) {
+            const float w = s < MAXS ? s_w[s] : weight(s);
+            if (w > 0.f) val = fmaf(p.part_o[(base + (int64_t)s * p.M) * D + d], w, val);
+        }
+        op[d] = SkLoad<T>::cvt(wsum > 0.f ? val / wsum : 0.f);
+    }
 }
 
 template <typename T, int D>
@@ -217,7 +243,7 @@ static hipError_t launch_splitk_t(const SplitKParams& p, hipStream_t stream) {
     else hipLaunchKernelGGL((splitk_partial_kernel<T, D, 1>), grid, dim3(SK_THREADS), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((splitk_merge_kernel<T, D>), dim3(p.M, p.H, p.B), dim3(D < 64 ? 64 : D), 0, stream, p);
+    hipLaunchKernelGGL((splitk_merge_kernel<T, D>), dim3(p.M, p.H, p.B), dim3(64), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -239,7 +265,7 @@ static hipError_t launch_merge_d(const SplitKParams& p, int D, hipStream_t s) {
         case 16: hipLaunchKernelGGL((splitk_merge_kernel<T, 16>), grid, dim3(64), 0, s, p); break;
         case 32: hipLaunchKernelGGL((splitk_merge_kernel<T, 32>), grid, dim3(64), 0, s, p); break;
         case 64: hipLaunchKernelGGL((splitk_merge_kernel<T, 64>), grid, dim3(64), 0, s, p); break;
-        case 128: hipLaunchKernelGGL((splitk_merge_kernel<T, 128>), grid, dim3(128), 0, s, p); break;
+        case 128: hipLaunchKernelGGL((splitk_merge_kernel<T, 128>), grid, dim3(64), 0, s, p); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
