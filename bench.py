@@ -33,7 +33,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel: rocprofv3 FETCH_SIZE and WRITE_SIZE, each scaled by what the
 # same counter reads for a 256 MiB device copy (profiles/fwd_kernel_bf16_d64_dense_B16_L1024.hbm_traffic.txt)
-MEASURED_TRAFFIC_BYTES = 1.0213e8
+MEASURED_TRAFFIC_BYTES = 1.0212e8
 B, H, L, D = 16, 12, 1024, 64
 
 
