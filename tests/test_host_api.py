@@ -96,6 +96,46 @@ def test_validation_without_gpu(lib):
     assert handle.t5a_splitk_workspace_bytes(2, 3, 1, 64, 4) == 2 * 3 * 4 * 1 * 66 * 4
 
 
+def test_workspace_sizes_and_checks_without_gpu(lib):
+    """sizes of the optional buffers, and the checks an entry point makes on them before any launch"""
+    handle = lib.load()
+    # distance LUTs: (H, 4, qlen) floats with qlen = 4 * (ceil((entries + 6) / 4) ... ) as the kernel lays them out
+    for causal, sat in ((0, 91), (1, 113)):           # saturation distances of 32 buckets / max_distance 128
+        entries = sat + 96 + (0 if causal else sat) + 96 + 1
+        qlen = 4 * ((entries + 6) // 4 + 1)
+        assert handle.t5a_bias_lut_bytes(12, 32, 128, causal) == 12 * 4 * qlen * 4
+    assert handle.t5a_bias_lut_bytes(12, 32, 4096, 0) == 0      # too long for the kernel's fetch: not offered
+    assert handle.t5a_bias_lut_bytes(0, 32, 128, 0) == 0
+    assert handle.t5a_bias_lut_bytes(12, 3, 128, 0) == 0        # bad bucket parameters
+    # launch plan of a packed batch: 64 bytes of counts, 8 lists of 2 * ceil(items / 8) entries of 32 bytes,
+    # 16 bytes per item for spilled entries; items = (total_q / 128 + B) * H
+    items = (70000 // 128 + 32) * 12
+    assert handle.t5a_varlen_workspace_bytes(32, 12, 70000) == 64 + 8 * 2 * ((items + 7) // 8) * 32 + items * 16
+    assert handle.t5a_varlen_workspace_bytes(2000, 12, 70000) == 0   # more sequences than the planner holds
+    assert handle.t5a_varlen_workspace_bytes(32, 12, 0) == 0
+    v = lib.T5AVarlenArgs()
+    v.dtype, v.B, v.H, v.D, v.total_q, v.total_k, v.max_seqlen_q, v.max_seqlen_k = 0, 32, 12, 64, 70000, 70000, 4096, 4096
+    v.q = v.k = v.v = v.o = v.cu_seqlens_q = v.cu_seqlens_k = 0x1000
+    for name in ("q_strides", "k_strides", "v_strides", "o_strides"):
+        setattr(v, name, (C.c_int64 * 2)(768, 64))
+    v.workspace, v.workspace_bytes = 0x2000, 100
+    assert handle.t5a_fwd_varlen(C.byref(v), None) == -8         # workspace too small
+    assert b"t5a_varlen_workspace_bytes" in handle.t5a_last_error()
+    v.workspace, v.workspace_bytes = 0x2004, 1 << 30
+    assert handle.t5a_fwd_varlen(C.byref(v), None) == -5         # workspace misaligned
+    d = lib.T5ADenseArgs()
+    d.dtype, d.B, d.H, d.M, d.N, d.D = 0, 1, 12, 128, 128, 64
+    d.q = d.k = d.v = d.o = 0x1000
+    for name in ("q_strides", "k_strides", "v_strides", "o_strides"):
+        setattr(d, name, (C.c_int64 * 3)(12 * 128 * 64, 128 * 64, 64))
+    d.bias.table, d.bias.table_dtype, d.bias.num_buckets, d.bias.max_distance = 0x3000, 1, 32, 128
+    d.bias.stride_bucket, d.bias.stride_head = 12, 1
+    d.bias.lut, d.bias.lut_bytes = 0x4000, 64
+    assert handle.t5a_fwd_dense(C.byref(d), None) == -8          # LUT buffer too small
+    d.bias.lut, d.bias.lut_bytes = 0x4008, 1 << 20
+    assert handle.t5a_fwd_dense(C.byref(d), None) == -5          # LUT buffer misaligned
+
+
 def test_ops_refuse_cpu_tensors():
     from turbot5_amd.ops import flash_attention_with_fusing_bias
     q = torch.zeros(1, 1, 8, 64)
