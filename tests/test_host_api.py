@@ -200,3 +200,24 @@ def test_packed_workload_lengths_fixture():
     assert fx["lengths"] == lens and fx["total"] == sum(lens)
     import bench
     assert bench.c3_lengths(torch) == lens
+
+
+def test_mask_info_is_not_inherited_by_another_tensor():
+    """The per-mask cache is keyed by address and version, which a new tensor can share with a freed one: an
+    entry only counts while the tensor it was made for is alive and is the one asked about."""
+    import gc
+    import weakref
+    from turbot5_amd import attentions as A
+    A._MASK_INFO.clear()
+    m = torch.tensor([[1, 1, 1, 0], [1, 0, 0, 0]])
+    all_ones, unpad = A._mask_info(m)
+    assert not all_ones and unpad[0] == "lens" and unpad[1][0].tolist() == [3, 1]
+    assert A._mask_info(m)[1] is unpad                      # same tensor: served from the cache
+    m2 = torch.tensor([[1, 1, 0, 0], [1, 1, 1, 1]])
+    key2 = (m2.data_ptr(), m2._version, tuple(m2.shape), str(m2.device), m2.dtype)
+    A._MASK_INFO[key2] = (weakref.ref(m), all_ones, unpad)   # what address reuse would leave behind
+    assert A._mask_info(m2)[1][1][0].tolist() == [2, 4]
+    ref = A._MASK_INFO[(m.data_ptr(), m._version, tuple(m.shape), str(m.device), m.dtype)][0]
+    del m
+    gc.collect()
+    assert ref() is None

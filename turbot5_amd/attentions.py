@@ -22,6 +22,7 @@ Differences from the reference, all on purpose:
 from __future__ import annotations
 
 import warnings
+import weakref
 from collections import OrderedDict
 from typing import Optional
 
@@ -70,10 +71,12 @@ _MASK_INFO: "OrderedDict[tuple, tuple]" = OrderedDict()
 
 
 def _mask_info(mask: torch.Tensor):
+    # The entry remembers WHICH tensor it describes (weakly): a later mask that happens to get the freed
+    # tensor's address, shape and version must not inherit its lengths.
     key = (mask.data_ptr(), mask._version, tuple(mask.shape), str(mask.device), mask.dtype)
     hit = _MASK_INFO.get(key)
-    if hit is not None:
-        return hit
+    if hit is not None and hit[0]() is mask:
+        return hit[1], hit[2]
     if mask.dim() != 2:
         raise ValueError(f"attention mask must be (batch, key_length) of 0/1, got shape {tuple(mask.shape)}")
     valid = mask != 0
@@ -93,7 +96,8 @@ def _mask_info(mask: torch.Tensor):
             unpad = ("lens", (lens, cu), {})
         else:
             unpad = ("packed", _get_unpad_data(valid.to(torch.int32)), {})
-    _MASK_INFO[key] = (all_ones, unpad)
+    _MASK_INFO[key] = (weakref.ref(mask), all_ones, unpad)
+    _MASK_INFO.move_to_end(key)
     while len(_MASK_INFO) > 16:
         _MASK_INFO.popitem(last=False)
     return all_ones, unpad
