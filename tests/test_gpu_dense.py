@@ -411,3 +411,44 @@ def test_bias_table_dtypes_and_layouts(gpu_device, tdtype, layout):
         finally:
             ops.BIAS_LUT_CACHE = True
         assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16], (cache, layout, tdtype)
+
+
+def test_packed_batch_with_a_shared_plan_under_graph_capture(gpu_device):
+    """A packed launch with a launch plan inside a device graph: the plan is rebuilt inside the graph (a plan
+    recorded during capture has not run, and one built before may be overwritten before a replay), so replays
+    follow the lengths that the captured cu_seqlens buffer holds at that moment.  The LaunchPlan object given
+    to the captured call is left untouched and still serves eager calls."""
+    from turbot5_amd.ops import LaunchPlan, flash_attention_with_fusing_bias_varlen
+    H, D, total = 4, 64, 30000
+    table = rnd(32, H, seed=303, scale=1.0).to(gpu_device)
+    sq, sk, sv = (torch.zeros(total, H, D, dtype=torch.bfloat16, device=gpu_device) for _ in range(3))
+    cu = torch.zeros(41, dtype=torch.int32, device=gpu_device)
+
+    def lengths(seed):
+        g = torch.Generator().manual_seed(seed)
+        cut = torch.sort(torch.randperm(total - 1, generator=g)[:39] + 1).values
+        return torch.cat([torch.tensor([0]), cut, torch.tensor([total])]).to(torch.int32)
+
+    cu.copy_(lengths(1))
+    plan = LaunchPlan()
+    call = lambda: flash_attention_with_fusing_bias_varlen(sq, sk, sv, table, cu, cu, total, total, causal=False,  # noqa: E731
+                                                           sm_scale=1.0, launch_plan=plan)
+    for _ in range(2):
+        call()                                               # builds the shared plan eagerly
+    torch.cuda.synchronize()
+    key = plan.key
+    assert key is not None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = call()
+    assert plan.key == key                                   # the capture did not touch the shared plan
+    for rep in range(3):
+        q, k, v = (rnd(total, H, D, seed=310 + 3 * rep + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+        new_cu = lengths(2 + rep).to(gpu_device)
+        eager = flash_attention_with_fusing_bias_varlen(q, k, v, table, new_cu, new_cu, total, total, causal=False,
+                                                        sm_scale=1.0, launch_plan=False)
+        torch.cuda.synchronize()
+        sq.copy_(q); sk.copy_(k); sv.copy_(v); cu.copy_(new_cu)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {rep} differs from the eager launch"

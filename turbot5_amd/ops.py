@@ -259,7 +259,8 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
         (launch_plan is True and items >= PLAN_MIN_ITEMS)
     ws_bytes = lib.t5a_varlen_workspace_bytes(B, H, total_q) if wanted else 0
     if ws_bytes > 0:
-        if isinstance(launch_plan, LaunchPlan):
+        # under graph capture nothing runs yet: a plan recorded there must not count as built for later eager calls
+        if shared and not torch.cuda.is_current_stream_capturing():
             key = tuple((t.data_ptr(), t._version) if t is not None else None for t in (cq, ck, lens[0], lens[1]))
             key += (B, H, D, total_q, a.dtype, a.causal, a.max_seqlen_q, a.max_seqlen_k, str(q.device))
             ws, ready = launch_plan.lookup(key, (cq, ck, lens[0], lens[1]), ws_bytes, q.device)
