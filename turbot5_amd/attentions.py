@@ -217,8 +217,8 @@ class T5FlashAttention(_T5AttentionBase):
             # one plan; other calls make their cu_q on the spot and plan per call
             plan = True
             if key_value_states is None and seq_length == key_length:
-                plan = plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt, seq_length),
-                                        ops.LaunchPlan())
+                plan = plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt, seq_length,
+                                         ops._stream(hidden_states)), ops.LaunchPlan())   # one per stream
             if kind == "lens":
                 # right-padded batch: the kernel walks the padded (B*L, H, D) layout with per-sequence
                 # lengths; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
