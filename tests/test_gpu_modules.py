@@ -103,6 +103,31 @@ def test_flash_encoder_with_left_padding_and_holes(gpu_device):
         assert (got[b][valid] - want).abs().max().item() <= 2e-3
 
 
+def test_flash_encoder_with_padding_on_either_side_runs_in_place(gpu_device):
+    """Rows that are one run of valid tokens (left padding, right padding, both, none, or no token at all) run
+    in place with a start row and a length per sequence; each sequence equals the oracle on its valid tokens
+    and the padded positions of the attention output are zero."""
+    from turbot5_amd import attentions as A
+    cfg, m, sd = make(dict(SMALL, attention_type="flash"))
+    ids = torch.randint(0, 200, (5, 150), generator=torch.Generator().manual_seed(6))
+    mask = torch.ones(5, 150)
+    mask[0, :40] = 0                 # left padding
+    mask[1, 90:] = 0                 # right padding
+    mask[2, :10] = 0
+    mask[2, 130:] = 0                # both
+    mask[4, :] = 0                   # nothing valid
+    dmask = mask.to(gpu_device)
+    assert A._mask_info(dmask)[1][0] == "lens"
+    m = m.to(gpu_device)
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), dmask).cpu()
+    for b in range(4):
+        valid = mask[b].bool()
+        want = OM.encoder_forward(sd, cfg, ids[b][valid][None])[0]
+        assert (got[b][valid] - want).abs().max().item() <= 2e-3, b
+    assert torch.isfinite(got).all()
+
+
 def test_bf16_attention_inside_fp32_model(gpu_device):
     cfg, m, sd = make(dict(SMALL, attention_type="flash", attention_dtype=torch.bfloat16))
     ids = torch.randint(0, 200, (2, 300), generator=torch.Generator().manual_seed(3))

@@ -82,17 +82,20 @@ def _mask_info(mask: torch.Tensor):
     valid = mask != 0
     lens = valid.sum(-1, dtype=torch.int32)
     steps = torch.arange(mask.shape[1], device=mask.device)
-    # one transfer for both questions: all ones?  right-padded (every row a run of ones, then zeros)?
-    all_ones, right_padded = (bool(x) for x in torch.stack(
-        [valid.all(), (valid == (steps[None, :] < lens[:, None])).all()]).tolist())
+    first = valid.to(torch.int8).argmax(-1)   # first valid token of a row (0 for an empty row)
+    # one transfer for both questions: all ones?  every row ONE run of ones (padding left, right or both)?
+    all_ones, one_run = (bool(x) for x in torch.stack(
+        [valid.all(), (valid == ((steps[None, :] >= first[:, None]) &
+                                 (steps[None, :] < (first + lens)[:, None]))).all()]).tolist())
     unpad = None
     if not all_ones:
-        # right-padded batches run in place with per-sequence lengths; anything else is packed first.
-        # The last element collects the launch plans of this batch, one per kind of attention call, so
-        # that the layers of a stack build each only once.
-        if right_padded:
+        # batches whose rows are one run of valid tokens run in place, with a start row and a length per
+        # sequence; anything else (holes) is packed first.  The last element collects the launch plans of
+        # this batch, one per kind of attention call, so that the layers of a stack build each only once.
+        if one_run:
             B, L = mask.shape
             cu = torch.arange(0, (B + 1) * L, L, dtype=torch.int32, device=mask.device)
+            cu[:B] += first.to(torch.int32)
             unpad = ("lens", (lens, cu), {})
         else:
             unpad = ("packed", _get_unpad_data(valid.to(torch.int32)), {})
@@ -220,8 +223,8 @@ class T5FlashAttention(_T5AttentionBase):
                 plan = plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt, seq_length,
                                          ops._stream(hidden_states)), ops.LaunchPlan())   # one per stream
             if kind == "lens":
-                # right-padded batch: the kernel walks the padded (B*L, H, D) layout with per-sequence
-                # lengths; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
+                # rows padded on either side: the kernel walks the padded (B*L, H, D) layout with a start row
+                # and a length per sequence; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
                 def rows(t, n):
                     t = t if t.is_contiguous() else t.contiguous()
                     return t.view(batch_size * n, self.n_heads, -1)
