@@ -563,6 +563,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // with K3 and V3.  Requests complete in order, so "at most K1 V1 K2 V2 outstanding" means that K0, V0,
     // Q and the column have landed: the LUT is built and the first product formed while the rest is in
     // flight.  (Q loaded into registers by the compiler would be waited for with "nothing outstanding".)
+    static_assert(!QDMA || (K_TILE * ES == 8192 && V_TILE * ES == 8192 && NSK == 4 && NSV == 4 && NTHREADS == 256),
+                  "the Q staging borrows 4 KB per wavefront from the last K and V ring stages");
     const unsigned q_stage = wave < 2 ? (unsigned)(NSV * V_TILE + 3 * K_TILE) * ES + wave * 4096u
                                       : (unsigned)(3 * V_TILE) * ES + (wave - 2) * 4096u;
     if constexpr (QDMA) {
