@@ -224,11 +224,13 @@ __global__ __launch_bounds__(PLAN_THREADS) void varlen_plan_kernel(const PlanPar
             s_stage[x * p.slots + s_nx[x] + (j - s_free[x])] = pack(it.x, it.y, it.z);
         }
         __syncthreads();
-        for (int x = 0; x < 8; ++x) {
+        {   // two wavefronts per XCD list, so that all lists are written at the same time
+            const int x = wave >> 1;
             const int room = max(0, p.slots - s_nx[x]);
             const int used = min(s_nx[x], p.slots) + min(room, max(0, n_over - s_free[x]));
             int4* list = reinterpret_cast<int4*>(p.plan) + ((x * p.slots) << 1);
-            for (int i = tid; i < 2 * used; i += PLAN_THREADS) {
+#pragma unroll 4
+            for (int i = (wave & 1) * 64 + lane; i < 2 * used; i += 128) {
                 const int w = s_stage[x * p.slots + (i >> 1)];
                 const int b = w & 1023;
                 list[i] = (i & 1) ? int4{s_lenk[b], s_qs[b], s_ks[b], 0}
