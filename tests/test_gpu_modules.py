@@ -182,3 +182,22 @@ def test_cross_attention_with_padded_memory(gpu_device):
     with torch.no_grad():
         logits, _, _ = m(ids.to(gpu_device), dec.to(gpu_device), attention_mask=mask.to(gpu_device))
     assert (logits.cpu() - want).abs().max().item() <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_relu_epilogue_path_equals_separate_relu(gpu_device, dtype):
+    """16-bit inference folds ReLU into wi's GEMM; the result must equal linear -> relu -> linear."""
+    from turbot5_amd import T5Config
+    from turbot5_amd.modeling import T5DenseActDense
+    torch.manual_seed(5)
+    ff = T5DenseActDense(T5Config(**SMALL)).to(gpu_device).to(dtype).eval()
+    assert "_zero_bias" not in ff.state_dict()
+    x = torch.randn(3, 70, 128, device=gpu_device).to(dtype)
+    with torch.no_grad():
+        got = ff(x)
+        want = ff.wo(torch.relu(ff.wi(x)))
+    assert got.shape == want.shape == (3, 70, 128)
+    assert (got.float() - want.float()).abs().max().item() <= 2e-2 * want.float().abs().max().item()
+    x.requires_grad_(True)      # with gradients wanted the layer takes the plain path
+    ff(x).sum().backward()
+    assert x.grad is not None

@@ -34,8 +34,19 @@ class T5DenseActDense(nn.Module):
         self.wi = nn.Linear(config.d_model, config.d_ff, bias=False)
         self.wo = nn.Linear(config.d_ff, config.d_model, bias=False)
         self.act = _ACT[config.dense_act_fn]
+        # a zero bias lets the GEMM library apply ReLU in the epilogue of wi (no separate pass over
+        # the (tokens, d_ff) activations); not part of the state_dict
+        self._relu = config.dense_act_fn == "relu"
+        self.register_buffer("_zero_bias", torch.zeros(config.d_ff), persistent=False)
 
     def forward(self, hidden_states):
+        w = self.wi.weight
+        if (self._relu and hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float16)
+                and w.dtype == hidden_states.dtype and self._zero_bias.dtype == w.dtype
+                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad))):
+            x = hidden_states.reshape(-1, hidden_states.shape[-1])
+            mid = torch._addmm_activation(self._zero_bias, x, w.t(), use_gelu=False)
+            return self.wo(mid).view(*hidden_states.shape[:-1], -1)
         return self.wo(self.act(self.wi(hidden_states)))
 
 
