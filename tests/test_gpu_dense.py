@@ -452,3 +452,27 @@ def test_packed_batch_with_a_shared_plan_under_graph_capture(gpu_device):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(captured, eager), f"replay {rep} differs from the eager launch"
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_scores_that_keep_climbing_along_the_keys(gpu_device, dtype, causal):
+    """The running row maximum has to be raised again and again: scores grow by 16 powers of two per
+    64 keys.  sm_scale = ln 2 makes the kernel's base-2 scaling of Q an identity and the ramp is a
+    small integer, so the scores themselves are exact and the usual tolerance applies."""
+    import math
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    B, H, L, D = 1, 2, 1500, 64
+    q, k, v = (rnd(B, H, L, D, seed=40 + i, dtype=dtype) for i in range(3))
+    q[..., 0] = 2.0
+    k[..., 0] = (torch.arange(L) // 16 * 2).to(dtype)
+    table = rnd(32, H, seed=43, scale=1.0)
+    sm = math.log(2.0)
+    out, lse = flash_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device),
+                                                causal=causal, sm_scale=sm, return_lse=True)
+    want = O.dense_attention(q, k, v, table, causal, sm)
+    want_lse = O.dense_lse(q, k, table, causal, sm)
+    tol = 5e-4 if dtype == torch.float32 else TOL[dtype]     # fp32: scores reach 250, one rounding of the scale shows
+    assert (out.float().cpu() - want).abs().max().item() <= tol
+    # the row sum adds probabilities as the matrix core sees them (rounded to the 16-bit type)
+    assert (lse.cpu() - want_lse).abs().max().item() <= (2e-3 if dtype == torch.float32 else 1e-2)

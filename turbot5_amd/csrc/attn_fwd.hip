@@ -110,7 +110,14 @@ constexpr int BM = 128;      // query rows per workgroup
 // tiles keep two workgroups per compute unit
 template <typename T, int D> constexpr int tile_keys() { return sizeof(T) == 2 && D == 128 ? 32 : 64; }
 constexpr int NTHREADS = 256;
-constexpr float kRaise = 8.0f;   // raise the running max only past 2^8
+// The running max of a row is raised only when a score exceeds it by more than this many powers of
+// two, so rows whose maximum creeps up over many tiles rescale their accumulators a few times, not on
+// every tile.  Probabilities then reach 2^limit: bf16 and fp32 have the exponent range for 2^24 (sums
+// and outputs are fp32 and are divided by the row sum at the end); fp16 tops out at 65504, hence 2^14.
+#ifndef T5A_RAISE
+#define T5A_RAISE 24.0f
+#endif
+template <typename T> constexpr float raise_limit() { return sizeof(T) == 2 && !__is_same(T, __bf16) ? 14.0f : T5A_RAISE; }
 #ifndef OCC
 #define OCC 2
 #endif
@@ -930,10 +937,10 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         // this lane's half of the row's keys; the other half sits in lane ^ 32 and is only consulted in the
         // rare block: "some lane of the wavefront must raise" is the same question for halves and for rows
         const float mh = max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3]));
-        if (__any((mh > kRaise) || (!started && mh > -INFINITY))) {
+        if (__any((mh > raise_limit<T>()) || (!started && mh > -INFINITY))) {
             asm volatile("");   // keep this rare block a real branch
             const float mx = xhalf_max(mh);
-            const bool raise = (mx > kRaise) || (!started && mx > -INFINITY);
+            const bool raise = (mx > raise_limit<T>()) || (!started && mx > -INFINITY);
             const float delta = raise ? mx : 0.f;
             const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
             m_run += delta;
