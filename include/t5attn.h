@@ -81,7 +81,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 103
+#define T5A_ABI_VERSION 104
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -226,12 +226,19 @@ int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
  * weight's type when that is 16 bit, else fp32 (torch type promotion of the reference code).
  * Arithmetic as the reference's eager path: fp32 variance and scaling, the scaled value rounded to
  * a 16-bit weight's type before the product; block sums are rounded to the input type first.
+ * residual (optional, group == 1 only): rows of x's type and shape with row stride
+ * residual_row_stride; the kernel normalises x + residual (rounded to x's type, as torch's add leaves
+ * it) and also writes that sum to sum_out (x's type, rows contiguous like y, 16-byte aligned; must
+ * not overlap x or residual).  This is the residual add of one T5 sub-layer followed by the norm of
+ * the next (src/turbot5/model/modeling.py:159-161, :113-114) in one pass over the rows.
  */
 typedef struct t5a_rmsnorm_args {
     const void* x; const void* weight; void* y;
     int64_t x_strides[2];
     int64_t batches; int32_t rows_per_batch; int32_t dim; int32_t group;
     int32_t x_dtype; int32_t weight_dtype; float eps;
+    int32_t reserved;
+    const void* residual; void* sum_out; int64_t residual_row_stride;
 } t5a_rmsnorm_args;
 int t5a_rmsnorm(const t5a_rmsnorm_args* args, t5a_stream_t stream);
 

@@ -71,3 +71,54 @@ def test_layer_norm_module_uses_the_kernel(gpu_device):
     got = m(x.to(gpu_device))
     assert got.dtype == torch.bfloat16
     assert (got.float().cpu() - want.float()).abs().max().item() <= 2.0 ** -6
+
+
+@pytest.mark.parametrize("xdt,wdt", [("bf16", "bf16"), ("f32", "f32"), ("f16", "f16"), ("f32", "bf16")])
+@pytest.mark.parametrize("shape", [(2, 100, 768), (1, 4096, 768), (3, 7, 512), (2, 9, 64), (2, 33, 4096), (1, 5, 2048)])
+def test_add_then_norm_in_one_kernel(gpu_device, xdt, wdt, shape):
+    """x + residual (rounded to x's type, exactly torch's add) and the norm of that sum; covers rows held
+    in registers (two and four chunks per lane) and the two-pass form (4096 columns)."""
+    from turbot5_amd.ops import rms_norm
+    g = torch.Generator().manual_seed(sum(shape) + len(xdt))
+    x = (2.0 * torch.randn(*shape, generator=g)).to(DT[xdt])
+    r = (1.5 * torch.randn(*shape, generator=g)).to(DT[xdt])
+    w = (1.0 + 0.2 * torch.randn(shape[-1], generator=g)).to(DT[wdt])
+    total, got = rms_norm(x.to(gpu_device), w.to(gpu_device), 1e-6, residual=r.to(gpu_device))
+    assert torch.equal(total.cpu(), x + r)                      # one correctly rounded add: bit-exact
+    want = O.rms_norm(x + r, w, 1e-6)
+    assert got.dtype == want.dtype and got.shape == want.shape and total.dtype == x.dtype
+    plain = rms_norm((x + r).to(gpu_device), w.to(gpu_device), 1e-6)
+    assert torch.equal(got, plain)                              # same arithmetic as the norm alone on the sum
+    diff = (got.float().cpu() - want.float()).abs()
+    ulp = {torch.float32: 1e-5, torch.bfloat16: 2.0 ** -6, torch.float16: 2.0 ** -9}[want.dtype]
+    assert (diff <= ulp * want.float().abs() + 2e-6).all()
+
+
+def test_add_norm_rejects_bad_arguments(gpu_device):
+    from turbot5_amd.ops import rms_norm
+    x = torch.randn(2, 8, 64, device=gpu_device)
+    w = torch.ones(64, device=gpu_device)
+    with pytest.raises(ValueError):
+        rms_norm(x, w, residual=x[:, :4])
+    with pytest.raises(ValueError):
+        rms_norm(x, w, group=2, residual=x)
+    with pytest.raises(ValueError):
+        rms_norm(x, w, residual=x.half())
+
+
+def test_layer_norm_add_norm_and_stack_equivalence(gpu_device):
+    """The stack hands each sub-layer's update to the next norm; block.forward adds it itself: same numbers."""
+    from turbot5_amd import T5Config, T5EncoderModel
+    torch.manual_seed(3)
+    cfg = T5Config(vocab_size=100, d_model=128, d_kv=64, d_ff=256, num_layers=2, num_heads=2, dropout_rate=0.0,
+                   attention_type="flash")
+    m = T5EncoderModel(cfg).eval().to(gpu_device).to(torch.bfloat16)
+    ids = torch.randint(0, 100, (2, 70), device=gpu_device)
+    with torch.no_grad():
+        got = m(ids)
+        h = m.shared(ids)
+        bias = None
+        for blk in m.encoder.block:
+            h, _, bias = blk(h, position_bias=bias)
+        want = m.encoder.final_layer_norm(h)
+    assert torch.equal(got, want)

@@ -62,6 +62,18 @@ class T5LayerNorm(nn.Module):
             x = x.to(self.weight.dtype)
         return self.weight * x
 
+    def add_norm(self, x: torch.Tensor, residual: Optional[torch.Tensor]):
+        """``(x + residual, norm(x + residual))``: the residual add that closes one sub-layer and the norm
+        that opens the next (reference src/turbot5/model/modeling.py:159-161, :113-114), one kernel on a
+        ROCm device.  ``residual`` None: ``(x, norm(x))``."""
+        if residual is None:
+            return x, self.forward(x)
+        if x.is_cuda and residual.dtype == x.dtype and not (torch.is_grad_enabled() and (x.requires_grad or residual.requires_grad)):
+            from .ops import rms_norm
+            return rms_norm(x, self.weight, self.eps, 1, residual)
+        total = x + residual
+        return total, self.forward(total)
+
 
 # ---------------------------------------------------------------------------------------------
 # One host synchronisation per distinct mask tensor (not per layer): is it all ones, and if not,

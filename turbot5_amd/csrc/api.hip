@@ -514,9 +514,17 @@ int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
     const int xunit = a->x_dtype == T5A_F32 ? 4 : 8;
     if (a->x_strides[0] % xunit != 0 || a->x_strides[1] % xunit != 0)
         return fail(T5A_ERR_STRIDE, "x strides must be multiples of %d elements", xunit);
+    if (a->residual != nullptr) {
+        if (a->group != 1) return fail(T5A_ERR_SHAPE, "a residual needs group == 1 (got %d)", a->group);
+        if (a->sum_out == nullptr) return fail(T5A_ERR_NULL, "residual given but sum_out is NULL");
+        if (!aligned16(a->residual) || !aligned16(a->sum_out) || a->residual_row_stride % xunit != 0 || a->residual_row_stride < 0)
+            return fail(T5A_ERR_STRIDE, "residual and sum_out must be 16-byte aligned, the residual row stride a multiple of %d elements", xunit);
+        if (a->sum_out == a->x || a->sum_out == a->residual) return fail(T5A_ERR_STRIDE, "sum_out must not overlap x or residual");
+    }
     RmsParams p;
     memset(&p, 0, sizeof(p));
     p.x = a->x; p.weight = a->weight; p.y = a->y;
+    p.residual = a->residual; p.sum_out = a->residual ? a->sum_out : nullptr; p.residual_row_stride = a->residual_row_stride;
     p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;
     p.out_per_batch = out_per_batch;
     p.out_rows = a->batches * out_per_batch;

@@ -1,9 +1,12 @@
 // T5 RMS norm (no mean subtraction, no bias) and the transient-global side-token producer
 // (block sums followed by the same norm) as one HBM-bound kernel.
 //
-// One wavefront per output row, four rows per workgroup.  A row is read twice (sum of squares,
-// then scale and store); the second read hits cache, so HBM sees one read and one write per
-// element.  Arithmetic follows the reference's eager path (src/turbot5/model/modules.py:51-59):
+// One wavefront per output row, four rows per workgroup.  Rows of up to 4 x 64 sixteen-byte chunks stay
+// in registers between the sum of squares and the scaling; longer rows are read twice (the second read
+// hits cache).  Either way HBM sees one read and one write per element.  With a residual the kernel
+// first forms x + residual (rounded to the input type, as torch's add leaves it), writes that sum out as
+// the new residual stream and normalises it: the "add, then norm" pair between two T5 sub-layers
+// (src/turbot5/model/modeling.py:159-161 followed by :113-114) as one pass.  Arithmetic follows the reference's eager path (src/turbot5/model/modules.py:51-59):
 // variance and normalisation in fp32, the normalised value rounded to the weight's type when that
 // is a 16-bit type, then multiplied by the weight in that type.  With group > 1 an output row is
 // the norm of the SUM of `group` consecutive input rows (rounded to the input type first, as the
@@ -31,8 +34,10 @@ template <> struct Cvt<_Float16> {
 
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 
-// TX input, TW weight, TY output (TY = TW for 16-bit weights, float otherwise)
-template <typename TX, typename TW, typename TY>
+// TX input, TW weight, TY output (TY = TW for 16-bit weights, float otherwise).
+// CH > 0: the row fits CH 16-byte chunks per lane and stays in registers between the sum of squares and
+// the scaling (one read of the row); CH == 0: any length, the row is read twice (the second read hits cache).
+template <typename TX, typename TW, typename TY, int CH>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     constexpr int VEC = 16 / sizeof(TX);   // elements per 16-byte load of the input
     const int lane = threadIdx.x & 63;
@@ -43,14 +48,23 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     const int first = g * p.group;
     const int count = g == p.out_per_batch - 1 ? p.rows_per_batch - first : p.group;
     const TX* x = reinterpret_cast<const TX*>(p.x) + b * p.x_batch_stride + (int64_t)first * p.x_row_stride;
+    const TX* res = p.residual ? reinterpret_cast<const TX*>(p.residual) + row * p.residual_row_stride : nullptr;
+    TX* sum = reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride;
     const TW* w = reinterpret_cast<const TW*>(p.weight);
     TY* y = reinterpret_cast<TY*>(p.y) + row * p.y_row_stride;
     const int nch = p.dim / VEC;
 
-    auto load = [&](int c, float (&f)[VEC]) {   // chunk c of the (summed) input row, as the input type holds it
+    // chunk c of the row to normalise, as the input type holds it: the input row, or the sum of `count`
+    // rows, or input + residual -- each sum rounded to the input type, as the torch expression leaves it
+    auto load = [&](int c, float (&f)[VEC]) {
         const Vec<TX, VEC> v = *reinterpret_cast<const Vec<TX, VEC>*>(x + c * VEC);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) f[i] = Cvt<TX>::up(v.v[i]);
+        if (res != nullptr) {
+            const Vec<TX, VEC> u = *reinterpret_cast<const Vec<TX, VEC>*>(res + c * VEC);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) f[i] = Cvt<TX>::up(Cvt<TX>::down(f[i] + Cvt<TX>::up(u.v[i])));
+        }
         if (count > 1) {
             for (int r = 1; r < count; ++r) {
                 const Vec<TX, VEC> u = *reinterpret_cast<const Vec<TX, VEC>*>(x + (int64_t)r * p.x_row_stride + c * VEC);
@@ -61,21 +75,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
             for (int i = 0; i < VEC; ++i) f[i] = Cvt<TX>::up(Cvt<TX>::down(f[i]));
         }
     };
-
-    float ss = 0.f;
-    for (int c = lane; c < nch; c += 64) {
-        float f[VEC];
-        load(c, f);
+    auto store = [&](int c, const float (&f)[VEC], float rs) {
+        if (res != nullptr) {   // the caller's new residual stream
+            Vec<TX, VEC> s;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) ss = fmaf(f[i], f[i], ss);
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-    const float rs = rsqrtf(ss / (float)p.dim + p.eps);
-
-    for (int c = lane; c < nch; c += 64) {
-        float f[VEC];
-        load(c, f);
+            for (int i = 0; i < VEC; ++i) s.v[i] = Cvt<TX>::down(f[i]);
+            *reinterpret_cast<Vec<TX, VEC>*>(sum + c * VEC) = s;
+        }
         Vec<TY, VEC> out;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -85,13 +91,55 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
             out.v[i] = Cvt<TY>::down(sizeof(TW) == 2 ? Cvt<TW>::up(Cvt<TW>::down(n)) * wi : n * wi);
         }
         *reinterpret_cast<Vec<TY, VEC>*>(y + c * VEC) = out;
+    };
+    auto wave_rsqrt = [&](float ss) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        return rsqrtf(ss / (float)p.dim + p.eps);
+    };
+
+    if constexpr (CH > 0) {
+        float f[CH][VEC];
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            const int c = lane + 64 * k;
+            if (c < nch) {
+                load(c, f[k]);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) ss = fmaf(f[k][i], f[k][i], ss);
+            }
+        }
+        const float rs = wave_rsqrt(ss);
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            const int c = lane + 64 * k;
+            if (c < nch) store(c, f[k], rs);
+        }
+    } else {
+        float ss = 0.f;
+        for (int c = lane; c < nch; c += 64) {
+            float f[VEC];
+            load(c, f);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) ss = fmaf(f[i], f[i], ss);
+        }
+        const float rs = wave_rsqrt(ss);
+        for (int c = lane; c < nch; c += 64) {
+            float f[VEC];
+            load(c, f);
+            store(c, f, rs);
+        }
     }
 }
 
 template <typename TX, typename TW, typename TY>
 static hipError_t launch_t(const RmsParams& p, hipStream_t s) {
     const unsigned grid = (unsigned)((p.out_rows + 3) / 4);
-    hipLaunchKernelGGL((rmsnorm_kernel<TX, TW, TY>), dim3(grid), dim3(256), 0, s, p);
+    const int per_lane = (p.dim / (16 / (int)sizeof(TX)) + 63) / 64;   // 16-byte chunks per lane
+    if (per_lane <= 2) hipLaunchKernelGGL((rmsnorm_kernel<TX, TW, TY, 2>), dim3(grid), dim3(256), 0, s, p);
+    else if (per_lane <= 4) hipLaunchKernelGGL((rmsnorm_kernel<TX, TW, TY, 4>), dim3(grid), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((rmsnorm_kernel<TX, TW, TY, 0>), dim3(grid), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -68,8 +68,15 @@ class T5LayerFF(nn.Module):
         self.DenseReluDense = T5DenseGatedActDense(config) if config.is_gated_act else T5DenseActDense(config)
         self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
+    def step(self, hidden_states, pending=None):
+        """(residual stream, this sub-layer's update): ``pending`` is the previous sub-layer's update, added
+        to the stream by the same kernel that norms it; the caller adds (or passes on) the returned update."""
+        hidden_states, normed = self.layer_norm.add_norm(hidden_states, pending)
+        return hidden_states, self.DenseReluDense(normed)
+
     def forward(self, hidden_states):
-        return hidden_states + self.DenseReluDense(self.layer_norm(hidden_states))
+        hidden_states, update = self.step(hidden_states)
+        return hidden_states + update
 
 
 class T5LayerSelfAttention(nn.Module):
@@ -85,14 +92,20 @@ class T5LayerSelfAttention(nn.Module):
             self.SelfAttention = cls(config, has_relative_attention_bias=has_relative_attention_bias)
         self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
-    def forward(self, hidden_states, attention_mask=None, position_bias=None, layer_head_mask=None,
-                past_key_value=None, use_cache=False, output_attentions=False):
-        normed = self.layer_norm(hidden_states)
+    def step(self, hidden_states, pending=None, attention_mask=None, position_bias=None, layer_head_mask=None,
+             past_key_value=None, use_cache=False, output_attentions=False):
+        """(residual stream, the attention module's tuple); element 0 of the tuple is the update to add."""
+        hidden_states, normed = self.layer_norm.add_norm(hidden_states, pending)
         kwargs = dict(mask=attention_mask, position_bias=position_bias, layer_head_mask=layer_head_mask,
                       past_key_value=past_key_value, output_attentions=output_attentions)
         if isinstance(self.SelfAttention, T5FlashAttention):
             kwargs["use_cache"] = use_cache
-        out = self.SelfAttention(normed, **kwargs)
+        return hidden_states, self.SelfAttention(normed, **kwargs)
+
+    def forward(self, hidden_states, attention_mask=None, position_bias=None, layer_head_mask=None,
+                past_key_value=None, use_cache=False, output_attentions=False):
+        hidden_states, out = self.step(hidden_states, None, attention_mask, position_bias, layer_head_mask,
+                                       past_key_value, use_cache, output_attentions)
         return (hidden_states + out[0],) + out[1:]
 
 
@@ -102,12 +115,17 @@ class T5LayerCrossAttention(nn.Module):
         self.EncDecAttention = T5FlashAttention(config, cross_attention=True, has_relative_attention_bias=False)
         self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
+    def step(self, hidden_states, pending, key_value_states, attention_mask=None, position_bias=None,
+             past_key_value=None, use_cache=False, query_length=None):
+        hidden_states, normed = self.layer_norm.add_norm(hidden_states, pending)
+        return hidden_states, self.EncDecAttention(normed, mask=attention_mask, key_value_states=key_value_states,
+                                                   position_bias=position_bias, past_key_value=past_key_value,
+                                                   use_cache=use_cache, query_length=query_length)
+
     def forward(self, hidden_states, key_value_states, attention_mask=None, position_bias=None,
                 past_key_value=None, use_cache=False, query_length=None):
-        normed = self.layer_norm(hidden_states)
-        out = self.EncDecAttention(normed, mask=attention_mask, key_value_states=key_value_states,
-                                   position_bias=position_bias, past_key_value=past_key_value,
-                                   use_cache=use_cache, query_length=query_length)
+        hidden_states, out = self.step(hidden_states, None, key_value_states, attention_mask, position_bias,
+                                       past_key_value, use_cache, query_length)
         return (hidden_states + out[0],) + out[1:]
 
 
@@ -120,22 +138,33 @@ class T5Block(nn.Module):
             self.layer.append(T5LayerCrossAttention(config))
         self.layer.append(T5LayerFF(config))
 
-    def forward(self, hidden_states, attention_mask=None, position_bias=None, encoder_hidden_states=None,
-                encoder_attention_mask=None, past_key_value=None, use_cache=False):
+    def step(self, hidden_states, pending=None, attention_mask=None, position_bias=None, encoder_hidden_states=None,
+             encoder_attention_mask=None, past_key_value=None, use_cache=False):
+        """The block with its last residual add left to the caller: returns (residual stream, update of the
+        feed-forward sub-layer, present, position_bias).  ``pending`` is the previous block's update.  Every
+        add between sub-layers happens inside the kernel that norms the sum for the next sub-layer."""
         self_past = past_key_value[:2] if past_key_value is not None else None
         cross_past = past_key_value[2:] if past_key_value is not None and len(past_key_value) == 4 else None
-        sa = self.layer[0](hidden_states, attention_mask=attention_mask, position_bias=position_bias,
-                           past_key_value=self_past, use_cache=use_cache)
-        hidden_states, present, position_bias = sa[0], sa[1], sa[2]
+        hidden_states, sa = self.layer[0].step(hidden_states, pending, attention_mask=attention_mask,
+                                               position_bias=position_bias, past_key_value=self_past,
+                                               use_cache=use_cache)
+        pending, present, position_bias = sa[0], sa[1], sa[2]
         if self.is_decoder and encoder_hidden_states is not None:
-            ca = self.layer[1](hidden_states, key_value_states=encoder_hidden_states,
-                               attention_mask=encoder_attention_mask, past_key_value=cross_past,
-                               use_cache=use_cache)
-            hidden_states = ca[0]
+            hidden_states, ca = self.layer[1].step(hidden_states, pending, key_value_states=encoder_hidden_states,
+                                                   attention_mask=encoder_attention_mask, past_key_value=cross_past,
+                                                   use_cache=use_cache)
+            pending = ca[0]
             if present is not None and ca[1] is not None:
                 present = present + ca[1]
-        hidden_states = self.layer[-1](hidden_states)
-        return hidden_states, present, position_bias
+        hidden_states, pending = self.layer[-1].step(hidden_states, pending)
+        return hidden_states, pending, present, position_bias
+
+    def forward(self, hidden_states, attention_mask=None, position_bias=None, encoder_hidden_states=None,
+                encoder_attention_mask=None, past_key_value=None, use_cache=False):
+        hidden_states, update, present, position_bias = self.step(
+            hidden_states, None, attention_mask, position_bias, encoder_hidden_states, encoder_attention_mask,
+            past_key_value, use_cache)
+        return hidden_states + update, present, position_bias
 
 
 class T5Stack(nn.Module):
@@ -160,13 +189,14 @@ class T5Stack(nn.Module):
         # the decoder's own padding mask has no meaning under causal attention with right padding;
         # only the encoder mask is routed down (as key padding of self- and cross-attention)
         self_mask = None if self.is_decoder else attention_mask
+        pending = None      # the last sub-layer's update, not yet added to the residual stream
         for blk, past in zip(self.block, past_key_values):
-            hidden_states, present, position_bias = blk(
-                hidden_states, attention_mask=self_mask, position_bias=position_bias,
+            hidden_states, pending, present, position_bias = blk.step(
+                hidden_states, pending, attention_mask=self_mask, position_bias=position_bias,
                 encoder_hidden_states=encoder_hidden_states, encoder_attention_mask=encoder_attention_mask,
                 past_key_value=past, use_cache=use_cache)
             presents.append(present)
-        hidden_states = self.final_layer_norm(hidden_states)
+        hidden_states = self.final_layer_norm.add_norm(hidden_states, pending)[1]
         return hidden_states, (presents if use_cache else None)
 
 

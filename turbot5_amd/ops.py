@@ -337,8 +337,13 @@ def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, b
                    NUM_BUCKETS, MAX_DISTANCE)
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1) -> torch.Tensor:
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1,
+             residual: Optional[torch.Tensor] = None):
     """T5 RMS norm over the last dimension (src/turbot5/model/modules.py:51-59).
+
+    With ``residual`` (same shape and dtype as x, group 1) the kernel normalises ``x + residual`` and
+    returns ``(x + residual, norm)``: the residual add that ends one T5 sub-layer and the norm that
+    opens the next (src/turbot5/model/modeling.py:159-161, :113-114) in one pass.
 
     ``group`` > 1: x is (B, L, d) and row r of the (B, L // group, d) result is the norm of the sum of
     rows [r*group, (r+1)*group) of its sequence, trailing rows joining the last group: the side-token
@@ -352,6 +357,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     out_dtype = weight.dtype if weight.dtype in (torch.float16, torch.bfloat16) else torch.float32
     w = weight.detach().contiguous()
     x_ = x.detach()
+    r2 = None
+    if residual is not None:
+        if group != 1 or residual.shape != x.shape or residual.dtype != x.dtype or residual.device != x.device:
+            raise ValueError("residual needs group == 1 and the shape, dtype and device of x")
+        r2 = residual.detach().reshape(-1, d)
+        if r2.stride(-1) != 1 or r2.stride(0) % 8 != 0 or r2.data_ptr() % 16 != 0:
+            r2 = r2.contiguous()
     if group == 1:
         x2 = x_.reshape(-1, d)
         if x2.stride(-1) != 1 or x2.stride(0) % 8 != 0 or x2.data_ptr() % 16 != 0:
@@ -372,9 +384,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     a.x_strides = (C.c_int64 * 2)(*strides)
     a.batches, a.rows_per_batch, a.dim, a.group = batches, rows, d, int(group)
     a.x_dtype, a.weight_dtype, a.eps = _dtype_code(x2), _dtype_code(w), float(eps)
+    total = None
+    if r2 is not None:
+        total = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        a.residual, a.sum_out, a.residual_row_stride = r2.data_ptr(), total.data_ptr(), r2.stride(0)
     with _on_device(x):
         L.check(L.load().t5a_rmsnorm(C.byref(a), _stream(x)))
-    return y
+    return y if total is None else (total, y)
 
 
 _CU_COUNT = {}
