@@ -184,9 +184,9 @@ def test_cross_attention_with_padded_memory(gpu_device):
     assert (logits.cpu() - want).abs().max().item() <= 5e-3
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_relu_epilogue_path_equals_separate_relu(gpu_device, dtype):
-    """16-bit inference folds ReLU into wi's GEMM; the result must equal linear -> relu -> linear."""
+    """Inference folds ReLU into wi's GEMM; the result must equal linear -> relu -> linear."""
     from turbot5_amd import T5Config
     from turbot5_amd.modeling import T5DenseActDense
     torch.manual_seed(5)

@@ -41,7 +41,8 @@ class T5DenseActDense(nn.Module):
 
     def forward(self, hidden_states):
         w = self.wi.weight
-        if (self._relu and hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float16)
+        if (self._relu and hasattr(torch, "_addmm_activation") and hidden_states.is_cuda
+                and hidden_states.dtype in (torch.bfloat16, torch.float16, torch.float32)
                 and w.dtype == hidden_states.dtype and self._zero_bias.dtype == w.dtype
                 and not (torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad))):
             x = hidden_states.reshape(-1, hidden_states.shape[-1])
