@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     const int count = g == p.out_per_batch - 1 ? p.rows_per_batch - first : p.group;
     const TX* x = reinterpret_cast<const TX*>(p.x) + b * p.x_batch_stride + (int64_t)first * p.x_row_stride;
     const TX* res = p.residual ? reinterpret_cast<const TX*>(p.residual) + row * p.residual_row_stride : nullptr;
-    TX* sum = reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride;
+    TX* sum = res ? reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride : nullptr;
     const TW* w = reinterpret_cast<const TW*>(p.weight);
     TY* y = reinterpret_cast<TY*>(p.y) + row * p.y_row_stride;
     const int nch = p.dim / VEC;
