@@ -201,3 +201,28 @@ def test_relu_epilogue_path_equals_separate_relu(gpu_device, dtype):
     x.requires_grad_(True)      # with gradients wanted the layer takes the plain path
     ff(x).sum().backward()
     assert x.grad is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gated_gelu_epilogue_path(gpu_device, dtype):
+    """'gated-gelu' (T5 v1.1): tanh-GELU in the epilogue of wi_0.  fp32 agrees to rounding; in bf16 the
+    epilogue rounds once (after the activation) where the separate kernels round twice."""
+    from turbot5_amd import T5Config
+    from turbot5_amd.modeling import T5DenseGatedActDense
+    torch.manual_seed(6)
+    cfg = T5Config(**dict(SMALL, feed_forward_proj="gated-gelu"))
+    assert cfg.dense_act_fn == "gelu_new" and cfg.is_gated_act
+    ff = T5DenseGatedActDense(cfg).to(gpu_device).to(dtype).eval()
+    assert "_zero_bias" not in ff.state_dict()
+    x = torch.randn(3, 70, 128, device=gpu_device).to(dtype)
+    with torch.no_grad():
+        got = ff(x)
+        want64 = (torch.nn.functional.gelu(x.double() @ ff.wi_0.weight.double().t(), approximate="tanh")
+                  * (x.double() @ ff.wi_1.weight.double().t())) @ ff.wo.weight.double().t()
+        plain = ff.wo(ff.act(ff.wi_0(x)) * ff.wi_1(x))
+    assert got.shape == (3, 70, 128)
+    scale = want64.abs().max().item()
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert (got.double() - want64).abs().max().item() <= tol * scale
+    # no worse than the separate kernels against exact arithmetic (a little slack for the different rounding)
+    assert (got.double() - want64).abs().max().item() <= 1.5 * (plain.double() - want64).abs().max().item() + 1e-6 * scale

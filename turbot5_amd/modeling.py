@@ -28,6 +28,15 @@ _ACT = {"relu": nn.functional.relu, "gelu": nn.functional.gelu, "silu": nn.funct
         "gelu_new": lambda x: nn.functional.gelu(x, approximate="tanh")}
 
 
+def _epilogue_ok(x, weight, zero_bias) -> bool:
+    """Inference on a ROCm device with one floating dtype throughout: the GEMM library can apply the
+    activation in the epilogue of the first projection (a private torch entry point, checked for)."""
+    return (hasattr(torch, "_addmm_activation") and x.is_cuda
+            and x.dtype in (torch.bfloat16, torch.float16, torch.float32)
+            and weight.dtype == x.dtype and zero_bias.dtype == x.dtype
+            and not (torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad)))
+
+
 class T5DenseActDense(nn.Module):
     def __init__(self, config: T5Config):
         super().__init__()
@@ -40,13 +49,9 @@ class T5DenseActDense(nn.Module):
         self.register_buffer("_zero_bias", torch.zeros(config.d_ff), persistent=False)
 
     def forward(self, hidden_states):
-        w = self.wi.weight
-        if (self._relu and hasattr(torch, "_addmm_activation") and hidden_states.is_cuda
-                and hidden_states.dtype in (torch.bfloat16, torch.float16, torch.float32)
-                and w.dtype == hidden_states.dtype and self._zero_bias.dtype == w.dtype
-                and not (torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad))):
+        if self._relu and _epilogue_ok(hidden_states, self.wi.weight, self._zero_bias):
             x = hidden_states.reshape(-1, hidden_states.shape[-1])
-            mid = torch._addmm_activation(self._zero_bias, x, w.t(), use_gelu=False)
+            mid = torch._addmm_activation(self._zero_bias, x, self.wi.weight.t(), use_gelu=False)
             return self.wo(mid).view(*hidden_states.shape[:-1], -1)
         return self.wo(self.act(self.wi(hidden_states)))
 
@@ -58,8 +63,16 @@ class T5DenseGatedActDense(nn.Module):
         self.wi_1 = nn.Linear(config.d_model, config.d_ff, bias=False)
         self.wo = nn.Linear(config.d_ff, config.d_model, bias=False)
         self.act = _ACT[config.dense_act_fn]
+        # tanh-GELU (the 'gated-gelu' of T5 v1.1 / Flan-T5) is the GEMM library's GELU epilogue: it is applied
+        # to the fp32 accumulator of wi_0 before the one rounding to the activation type
+        self._gelu_tanh = config.dense_act_fn == "gelu_new"
+        self.register_buffer("_zero_bias", torch.zeros(config.d_ff), persistent=False)
 
     def forward(self, hidden_states):
+        if self._gelu_tanh and _epilogue_ok(hidden_states, self.wi_0.weight, self._zero_bias):
+            x = hidden_states.reshape(-1, hidden_states.shape[-1])
+            gate = torch._addmm_activation(self._zero_bias, x, self.wi_0.weight.t(), use_gelu=True)
+            return self.wo(gate * self.wi_1(x)).view(*hidden_states.shape[:-1], -1)
         return self.wo(self.act(self.wi_0(hidden_states)) * self.wi_1(hidden_states))
 
 
