@@ -162,8 +162,8 @@ def extra_workloads(torch, dev, steps, full):
         f = lambda: enc16(ids)  # noqa: E731
         _, ms = time_kernel(torch, f, 5, 2)
         out["t5_base_encoder_8k_B2_bf16"] = {"ms": round(ms, 2), "tokens_per_s": round(2 * 8192 / (ms * 1e-3), 1)}
-        # a padded batch: 16 rows of 4096 positions, 128..4096 valid tokens each (right padding); the attention
-        # runs in place on the padded layout with one launch plan shared by the 12 layers
+        # a padded batch: 16 rows of 4096 positions, 128..4096 valid tokens each (right padding); the stack packs
+        # the valid tokens once and runs all 12 layers on them, with one launch plan shared by the layers
         plens = torch.randint(128, 4097, (16,), generator=torch.Generator().manual_seed(2))
         pmask = (torch.arange(4096)[None, :] < plens[:, None]).to(torch.float32).to(dev)
         ids = torch.randint(0, 32128, (16, 4096), generator=ids_g).to(dev)

@@ -226,3 +226,45 @@ def test_gated_gelu_epilogue_path(gpu_device, dtype):
     assert (got.double() - want64).abs().max().item() <= tol * scale
     # no worse than the separate kernels against exact arithmetic (a little slack for the different rounding)
     assert (got.double() - want64).abs().max().item() <= 1.5 * (plain.double() - want64).abs().max().item() + 1e-6 * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_encoder_runs_padded_batches_on_their_valid_tokens(gpu_device, dtype):
+    """The stack packs the valid tokens once and runs every layer on them; with the switch off it keeps
+    the padded layout (attention in place or gather/scatter per layer).  Same numbers at the valid
+    positions, zeros at the padded ones; masks with holes, padding on both sides and an empty row."""
+    cfg, m, sd = make(dict(SMALL, attention_type="flash"))
+    ids = torch.randint(0, 200, (5, 150), generator=torch.Generator().manual_seed(8))
+    for case in ("one run", "holes"):
+        mask = torch.ones(5, 150)
+        mask[0, :40] = 0
+        mask[1, 90:] = 0
+        mask[2, :10] = 0
+        mask[2, 130:] = 0
+        mask[4, :] = 0
+        if case == "holes":
+            mask[3, 20:25] = 0
+        m = m.to(gpu_device).to(dtype)
+        dmask = mask.to(gpu_device)
+        assert m.encoder.pack_padded_batches
+        with torch.no_grad():
+            got = m(ids.to(gpu_device), dmask)
+            m.encoder.pack_padded_batches = False
+            ref = m(ids.to(gpu_device), dmask)
+            m.encoder.pack_padded_batches = True
+        valid = mask.bool()
+        tol = 1e-5 if dtype == torch.float32 else 3e-2
+        assert (got.float().cpu()[valid] - ref.float().cpu()[valid]).abs().max().item() <= tol
+        assert (got.cpu()[~valid] == 0).all()
+        if dtype == torch.float32:
+            for b in range(4):
+                want = OM.encoder_forward(sd, cfg, ids[b][valid[b]][None])[0]
+                assert (got.cpu()[b][valid[b]] - want).abs().max().item() <= 2e-3, (case, b)
+
+
+def test_packed_stack_is_off_for_decoders_and_sparse_types(gpu_device):
+    from turbot5_amd import T5Config, T5EncoderModel, T5Model
+    enc = T5EncoderModel(T5Config(**dict(SMALL, attention_type="local", sliding_window=64)))
+    assert not enc.encoder.pack_padded_batches
+    full = T5Model(T5Config(**dict(SMALL, attention_type="flash")))
+    assert full.encoder.pack_padded_batches and not full.decoder.pack_padded_batches

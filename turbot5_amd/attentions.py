@@ -118,6 +118,31 @@ def _mask_info(mask: torch.Tensor):
     return all_ones, unpad
 
 
+class PackedBatch:
+    """The valid tokens of a padded (B, L) batch laid back to back: what a whole layer stack needs to run
+    on ``total`` rows instead of ``B * L`` (the reference packs and pads around every attention call,
+    attentions.py:492-511, and runs everything else on the padded rows)."""
+    __slots__ = ("indices", "cu_seqlens", "max_len", "batch", "length", "plans")
+
+    def __init__(self, indices, cu_seqlens, max_len, batch, length, plans):
+        self.indices, self.cu_seqlens, self.max_len = indices, cu_seqlens, max_len
+        self.batch, self.length, self.plans = batch, length, plans
+
+
+def packed_batch(mask: torch.Tensor) -> Optional[PackedBatch]:
+    """None for an all-ones mask; otherwise the packed layout of its valid tokens, remembered with the
+    mask (one more host synchronisation per distinct mask tensor: the number of valid tokens)."""
+    all_ones, unpad = _mask_info(mask)
+    if all_ones:
+        return None
+    kind, data, plans = unpad
+    hit = plans.get("packed_batch")
+    if hit is None:
+        indices, cu, max_len = data if kind == "packed" else _get_unpad_data((mask != 0).to(torch.int32))
+        hit = plans["packed_batch"] = PackedBatch(indices, cu, max_len, mask.shape[0], mask.shape[1], {})
+    return hit
+
+
 class _T5AttentionBase(nn.Module):
     """Parameters and shape helpers shared by the attention modules (attentions.py:36-66)."""
 
@@ -274,6 +299,23 @@ class T5FlashAttention(_T5AttentionBase):
         attn_output = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
         present_key_value_state = (key_states, value_states) if (self.is_decoder and use_cache) else None
         return (attn_output,) + (present_key_value_state,) + (table,)
+
+    def forward_packed(self, hidden_states, packed: PackedBatch, position_bias=None):
+        """Self-attention over hidden states that are already packed: (total, d_model), sequences back to
+        back as ``packed.cu_seqlens`` says.  No gather, no scatter; positions count the tokens of a
+        sequence, as in the reference's packed call (varlen_fused_bias_attn.py:254, :303)."""
+        total = hidden_states.shape[0]
+        adt = self._attn_dtype(hidden_states)
+        q, k, v = (p(hidden_states).view(total, self.n_heads, self.key_value_proj_dim).to(adt)
+                   for p in (self.q, self.k, self.v))
+        table = self._table(position_bias)
+        plan = packed.plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt,
+                                        ops._stream(hidden_states)), ops.LaunchPlan())
+        out = ops.flash_attention_with_fusing_bias_varlen(
+            q, k, v, table, packed.cu_seqlens, packed.cu_seqlens, packed.max_len, packed.max_len,
+            causal=self.causal, sm_scale=1.0, NUM_BUCKETS=self.relative_attention_num_buckets,
+            MAX_DISTANCE=self.relative_attention_max_distance, launch_plan=plan)
+        return (self.o(out.reshape(total, self.inner_dim).to(hidden_states.dtype)), None, table)
 
 
 class _SparseBase(_T5AttentionBase):

@@ -21,7 +21,8 @@ from typing import List, Optional, Tuple
 import torch
 from torch import nn
 
-from .attentions import T5ATTENTION_TYPES, T5FlashAttention, T5LayerNorm
+from .attentions import T5ATTENTION_TYPES, T5FlashAttention, T5LayerNorm, packed_batch
+from .padding import index_first_axis, pad_input
 from .config import T5Config
 
 _ACT = {"relu": nn.functional.relu, "gelu": nn.functional.gelu, "silu": nn.functional.silu,
@@ -107,9 +108,12 @@ class T5LayerSelfAttention(nn.Module):
         self.layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
     def step(self, hidden_states, pending=None, attention_mask=None, position_bias=None, layer_head_mask=None,
-             past_key_value=None, use_cache=False, output_attentions=False):
-        """(residual stream, the attention module's tuple); element 0 of the tuple is the update to add."""
+             past_key_value=None, use_cache=False, output_attentions=False, packed=None):
+        """(residual stream, the attention module's tuple); element 0 of the tuple is the update to add.
+        ``packed``: the hidden states are the packed valid tokens of a padded batch (flash attention only)."""
         hidden_states, normed = self.layer_norm.add_norm(hidden_states, pending)
+        if packed is not None:
+            return hidden_states, self.SelfAttention.forward_packed(normed, packed, position_bias)
         kwargs = dict(mask=attention_mask, position_bias=position_bias, layer_head_mask=layer_head_mask,
                       past_key_value=past_key_value, output_attentions=output_attentions)
         if isinstance(self.SelfAttention, T5FlashAttention):
@@ -153,7 +157,7 @@ class T5Block(nn.Module):
         self.layer.append(T5LayerFF(config))
 
     def step(self, hidden_states, pending=None, attention_mask=None, position_bias=None, encoder_hidden_states=None,
-             encoder_attention_mask=None, past_key_value=None, use_cache=False):
+             encoder_attention_mask=None, past_key_value=None, use_cache=False, packed=None):
         """The block with its last residual add left to the caller: returns (residual stream, update of the
         feed-forward sub-layer, present, position_bias).  ``pending`` is the previous block's update.  Every
         add between sub-layers happens inside the kernel that norms the sum for the next sub-layer."""
@@ -161,7 +165,7 @@ class T5Block(nn.Module):
         cross_past = past_key_value[2:] if past_key_value is not None and len(past_key_value) == 4 else None
         hidden_states, sa = self.layer[0].step(hidden_states, pending, attention_mask=attention_mask,
                                                position_bias=position_bias, past_key_value=self_past,
-                                               use_cache=use_cache)
+                                               use_cache=use_cache, packed=packed)
         pending, present, position_bias = sa[0], sa[1], sa[2]
         if self.is_decoder and encoder_hidden_states is not None:
             hidden_states, ca = self.layer[1].step(hidden_states, pending, key_value_states=encoder_hidden_states,
@@ -190,6 +194,14 @@ class T5Stack(nn.Module):
         n = config.num_decoder_layers if config.is_decoder else config.num_layers
         self.block = nn.ModuleList([T5Block(config, has_relative_attention_bias=bool(i == 0)) for i in range(n)])
         self.final_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
+        # An encoder with full ('flash') attention runs a padded batch on its valid tokens only: they are
+        # packed once after the embedding, every layer (projections, attention through cu_seqlens, norms,
+        # feed-forward) works on (total, d_model), and the result is scattered back into zeros at the end.
+        # The reference packs and pads around each attention call only (attentions.py:492-511) and spends
+        # the dense layers on the padding too.  Outputs at valid positions are the same; padded positions
+        # of the result are zero.  Set to False to keep the padded layout through the stack.
+        self.pack_padded_batches = (not config.is_decoder) and all(
+            isinstance(b.layer[0].SelfAttention, T5FlashAttention) for b in self.block)
 
     def forward(self, input_ids=None, attention_mask=None, encoder_hidden_states=None, encoder_attention_mask=None,
                 inputs_embeds=None, past_key_values=None, use_cache=False):
@@ -203,14 +215,23 @@ class T5Stack(nn.Module):
         # the decoder's own padding mask has no meaning under causal attention with right padding;
         # only the encoder mask is routed down (as key padding of self- and cross-attention)
         self_mask = None if self.is_decoder else attention_mask
+        packed = None
+        if self.pack_padded_batches and self_mask is not None and hidden_states.is_cuda:
+            packed = packed_batch(self_mask)
+            if packed is not None and packed.indices.numel() == 0:
+                packed = None       # nothing valid anywhere: the padded route handles empty sequences
+            if packed is not None:
+                hidden_states = index_first_axis(hidden_states.reshape(-1, hidden_states.shape[-1]), packed.indices)
         pending = None      # the last sub-layer's update, not yet added to the residual stream
         for blk, past in zip(self.block, past_key_values):
             hidden_states, pending, present, position_bias = blk.step(
                 hidden_states, pending, attention_mask=self_mask, position_bias=position_bias,
                 encoder_hidden_states=encoder_hidden_states, encoder_attention_mask=encoder_attention_mask,
-                past_key_value=past, use_cache=use_cache)
+                past_key_value=past, use_cache=use_cache, packed=packed)
             presents.append(present)
         hidden_states = self.final_layer_norm.add_norm(hidden_states, pending)[1]
+        if packed is not None:
+            hidden_states = pad_input(hidden_states, packed.indices, packed.batch, packed.length)
         return hidden_states, (presents if use_cache else None)
 
 
