@@ -81,7 +81,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 104
+#define T5A_ABI_VERSION 105
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -172,6 +172,10 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           reference computes them, attentions.py:722-732, :807-814).
  *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
  *           (B,H,n_side,D) projected block aggregates, bias bucket(g - min(i/aux, n_side-1)).
+ * seq_lens (optional, LOCAL only): (B) int32 on the device, the number of valid tokens of each
+ * right-padded sequence.  Keys at or past a sequence's length are not attended (the key half of the
+ * reference's local mask, src/turbot5/model/utils.py:174-188); rows past the length are still
+ * written (from the keys left in their window, zeros when there are none) and mean nothing.
  * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
  * the G global rows, which attend all L keys, are computed as key splits spread over the whole
  * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
@@ -187,6 +191,7 @@ typedef struct t5a_sparse_args {
     int32_t pattern; int32_t block_len; int32_t aux; int32_t n_side;
     float sm_scale; int32_t reserved;
     t5a_bias bias;
+    const int32_t* seq_lens;
 } t5a_sparse_args;
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux);
 int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);

@@ -56,7 +56,7 @@ def basic_self_attention(sd: SD, prefix: str, cfg, hidden: torch.Tensor, table: 
             bias = bias + torch.where(key_mask[:, None, None, :] > 0, 0.0, float("-inf"))
         out = torch.nan_to_num(O.basic_attention(q, k, v, bias), nan=0.0)
     elif attention_type == "local":
-        out = O.local_attention_blocked(q, k, v, table, cfg.sliding_window, None, nb, md)
+        out = O.local_attention_blocked(q, k, v, table, cfg.sliding_window, key_mask, nb, md)
     elif attention_type == "block":
         out = O.block_attention_blocked(q, k, v, table, cfg.sliding_window, cfg.global_block_size, None, nb, md)
     elif attention_type == "transient-global":

@@ -61,9 +61,13 @@ def test_attention_module_output_tuple(gpu_device):
         with torch.no_grad():
             out2 = later(x, position_bias=out[2])
         assert out2[0].shape == (2, 96, 128)
-    with pytest.raises(NotImplementedError):
-        mask = torch.ones(2, 96, device=gpu_device)
-        mask[1, 50:] = 0
+    mask = torch.ones(2, 96, device=gpu_device)
+    mask[1, 50:] = 0
+    for name in ("block", "transient-global"):       # right padding is the local pattern's only
+        with pytest.raises(NotImplementedError):
+            T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
+    mask[0, :3] = 0
+    with pytest.raises(NotImplementedError):         # left padding
         T5ATTENTION_TYPES["local"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
 
 
@@ -268,3 +272,22 @@ def test_packed_stack_is_off_for_decoders_and_sparse_types(gpu_device):
     assert not enc.encoder.pack_padded_batches
     full = T5Model(T5Config(**dict(SMALL, attention_type="flash")))
     assert full.encoder.pack_padded_batches and not full.decoder.pack_padded_batches
+
+
+def test_local_encoder_with_right_padding(gpu_device):
+    """T5LocalAttention takes right-padded batches (per-sequence key limit in the kernel); other masks raise."""
+    cfg, m, sd = make(dict(SMALL, attention_type="local", sliding_window=64))
+    ids = torch.randint(0, 200, (3, 256), generator=torch.Generator().manual_seed(9))
+    mask = torch.ones(3, 256)
+    mask[0, 200:] = 0
+    mask[2, 30:] = 0
+    want = OM.encoder_forward(sd, cfg, ids, mask, attention_type="local")
+    m = m.to(gpu_device)
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
+    valid = mask.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+    left = torch.ones(3, 256)
+    left[1, :10] = 0
+    with pytest.raises(NotImplementedError), torch.no_grad():
+        m(ids.to(gpu_device), left.to(gpu_device))

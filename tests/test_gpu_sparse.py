@@ -128,3 +128,38 @@ def test_splitk_with_bias_and_head_dims(gpu_device):
         s = torch.einsum("bhqd,bhkd->bhqk", q * 0.8, k) + bias
         want = torch.softmax(s, -1) @ v
         assert (res.cpu() - want).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,lens", [(512, 128, [512, 300, 1, 129]), (384, 64, [100, 0, 384, 63]),
+                                       (256, 16, [255, 17, 16, 200]), (1024, 512, [700, 1024, 511, 5])])
+def test_local_with_sequence_lengths(gpu_device, dtype, L, Bl, lens):
+    """Right-padded batch through the local pattern: valid rows equal the oracle's mask path
+    (key valid and query valid and inside the window, utils.py:174-188)."""
+    from turbot5_amd.ops import local_attention_with_fusing_bias
+    B, H, D = len(lens), 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=60 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=63, scale=1.0)
+    mask = (torch.arange(L)[None, :] < torch.tensor(lens)[:, None]).float()
+    out = local_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device), Bl,
+                                           seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu_device))
+    want = O.local_attention_blocked(q, k, v, table, Bl, mask)
+    assert torch.isfinite(out).all()
+    for b, n in enumerate(lens):
+        if n:
+            assert (out.float().cpu()[b, :, :n] - want[b, :, :n]).abs().max().item() <= TOL[dtype], (b, n)
+    # full lengths: the same numbers as the call without lengths
+    full = torch.full((B,), L, dtype=torch.int32, device=gpu_device)
+    a = local_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device), Bl, seq_lens=full)
+    b_ = local_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device), Bl)
+    assert torch.equal(a, b_)
+
+
+def test_sequence_lengths_are_for_the_local_pattern_only(gpu_device):
+    from turbot5_amd import ops
+    q = torch.zeros(1, 1, 128, 64, device=gpu_device, dtype=torch.bfloat16)
+    lens = torch.tensor([100], dtype=torch.int32, device=gpu_device)
+    with pytest.raises(ValueError):
+        ops._sparse(ops.L.PATTERN_BLOCK, q, q, q, None, 64, 16, seq_lens=lens)
+    with pytest.raises(ValueError):
+        ops.local_attention_with_fusing_bias(q, q, q, None, 64, seq_lens=lens.long())

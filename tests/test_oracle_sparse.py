@@ -81,6 +81,46 @@ def test_local_against_huggingface(hf, L, Bl):
     assert torch.allclose(got, want, atol=2e-5)
 
 
+@pytest.mark.parametrize("L,Bl", [(64, 16), (96, 32)])
+def test_local_with_padding_against_huggingface(hf, L, Bl):
+    """Right-padded batch: the oracle's mask path against LongT5LocalAttention with the same mask,
+    compared on the valid query rows (padded rows attend a uniformly masked window in both)."""
+    B, H, D = 3, 2, 8
+    mod = hf.LongT5LocalAttention(_hf_cfg(hf, H, D, Bl), has_relative_attention_bias=True).eval()
+    table = rnd(32, H, seed=24, scale=1.0)
+    am = torch.ones(B, L)
+    am[0, L - 5:] = 0
+    am[1, Bl + 3:] = 0
+    with torch.no_grad():
+        mod.relative_attention_bias.weight.copy_(table)
+        mod.o.weight.copy_(torch.eye(H * D))
+        x = rnd(B, L, H * D, seed=25, scale=1.0)
+        want = mod(x, mask=hf._get_local_attention_mask(am, Bl, x.device))[0]
+        q = mod.q(x).view(B, L, H, D).transpose(1, 2)
+        k = mod.k(x).view(B, L, H, D).transpose(1, 2)
+        v = mod.v(x).view(B, L, H, D).transpose(1, 2)
+    got = O.local_attention_blocked(q, k, v, table, Bl, am).transpose(1, 2).reshape(B, L, H * D)
+    valid = am.bool()
+    assert torch.allclose(got[valid], want[valid], atol=2e-5)
+
+
+def test_local_with_padding_against_brute_force():
+    """Valid rows of a right-padded batch equal plain attention over the valid keys inside the window."""
+    B, H, L, D, Bl = 2, 2, 48, 4, 16
+    q, k, v = (rnd(B, H, L, D, seed=26 + i) for i in range(3))
+    table = rnd(32, H, seed=29, scale=1.0)
+    lens = [37, 9]
+    am = (torch.arange(L)[None, :] < torch.tensor(lens)[:, None]).float()
+    got = O.local_attention_blocked(q, k, v, table, Bl, am)
+    i = torch.arange(L)[:, None]
+    j = torch.arange(L)[None, :]
+    bias = table[O.relative_position_bucket(j - i, True, 32, 128)].permute(2, 0, 1).unsqueeze(0)
+    for b, n in enumerate(lens):
+        keep = ((j - i).abs() < Bl) & (j < n)
+        want = O.basic_attention(q[b:b + 1], k[b:b + 1], v[b:b + 1], bias.masked_fill(~keep, float("-inf")))
+        assert (got[b, :, :n] - want[0, :, :n]).abs().max().item() < 2e-6
+
+
 @pytest.mark.parametrize("L,Bl", [(40, 8), (48, 16), (8, 8), (5, 8)])
 def test_local_against_closed_form(L, Bl):
     H, D = 2, 4

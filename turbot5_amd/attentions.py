@@ -96,9 +96,10 @@ def _mask_info(mask: torch.Tensor):
     steps = torch.arange(mask.shape[1], device=mask.device)
     first = valid.to(torch.int8).argmax(-1)   # first valid token of a row (0 for an empty row)
     # one transfer for both questions: all ones?  every row ONE run of ones (padding left, right or both)?
-    all_ones, one_run = (bool(x) for x in torch.stack(
+    all_ones, one_run, from_zero = (bool(x) for x in torch.stack(
         [valid.all(), (valid == ((steps[None, :] >= first[:, None]) &
-                                 (steps[None, :] < (first + lens)[:, None]))).all()]).tolist())
+                                 (steps[None, :] < (first + lens)[:, None]))).all(),
+         (first == 0).all()]).tolist())
     unpad = None
     if not all_ones:
         # batches whose rows are one run of valid tokens run in place, with a start row and a length per
@@ -108,7 +109,7 @@ def _mask_info(mask: torch.Tensor):
             B, L = mask.shape
             cu = torch.arange(0, (B + 1) * L, L, dtype=torch.int32, device=mask.device)
             cu[:B] += first.to(torch.int32)
-            unpad = ("lens", (lens, cu), {})
+            unpad = ("lens", (lens, cu), {"right_padded": from_zero})
         else:
             unpad = ("packed", _get_unpad_data(valid.to(torch.int32)), {})
     _MASK_INFO[key] = (weakref.ref(mask), all_ones, unpad)
@@ -319,18 +320,24 @@ class T5FlashAttention(_T5AttentionBase):
 
 
 class _SparseBase(_T5AttentionBase):
-    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions):
+    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions,
+                    right_padding_ok=False):
+        """Returns the (B,) int32 lengths of a right-padded batch when the pattern supports them, else None."""
         if past_key_value is not None:
             warnings.warn('Currently, passing past key value states is not supported.')
         if use_cache is not None:
             warnings.warn('Currently, using cache is not supported for chosen attention type.')
         self._reject(layer_head_mask, output_attentions)
         if mask is not None:
-            all_ones, _ = _mask_info(mask)
+            all_ones, unpad = _mask_info(mask)
             if not all_ones:
+                if right_padding_ok and unpad[0] == "lens" and unpad[2].get("right_padded"):
+                    return unpad[1][0]
                 raise NotImplementedError(
-                    f"{type(self).__name__} runs as tile skipping for all-ones attention masks only; "
-                    "use attention_type='flash' for padded batches")
+                    f"{type(self).__name__} runs as tile skipping for all-ones attention masks"
+                    + (" and right-padded batches" if right_padding_ok else "")
+                    + " only; use attention_type='flash' for other padded batches")
+        return None
 
     def _qkv(self, hidden_states):
         batch_size = hidden_states.shape[0]
@@ -352,14 +359,17 @@ class T5LocalAttention(_SparseBase):
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
-        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        # right-padded batches: the keys of a sequence end at its length (the key half of the reference's
+        # local mask, utils.py:174-188); outputs at padded positions mean nothing, as in the reference
+        seq_lens = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
+                                    right_padding_ok=True)
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
         # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
         block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.local_attention_with_fusing_bias(
             q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance)
+            self.relative_attention_max_distance, seq_lens=seq_lens)
         return self._finish(out, hidden_states, table)
 
 

@@ -402,6 +402,10 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.sk_sb = a->side_k_strides[0]; p.sk_sh = a->side_k_strides[1]; p.sk_sr = a->side_k_strides[2];
     p.sv_sb = a->side_v_strides[0]; p.sv_sh = a->side_v_strides[1]; p.sv_sr = a->side_v_strides[2];
     p.B = a->B; p.H = a->H; p.M = a->L; p.N = a->L;
+    if (a->seq_lens != nullptr) {
+        if (a->pattern != T5A_PATTERN_LOCAL) return fail(T5A_ERR_PATTERN, "seq_lens is supported by the local pattern only");
+        p.len_k = a->seq_lens;
+    }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
     p.c1 = a->sm_scale * kLog2e;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;

@@ -356,6 +356,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         h = (int)(bh - (unsigned)b * (unsigned)p.H);
         Mseq = p.M;
         Nseq = p.N;
+        // local pattern on a right-padded batch: the keys of a sequence end at its length; positions are
+        // the row indices, so nothing else changes (rows past the length see what is left of their window)
+        if (MODE == kLocal && p.len_k != nullptr) Nseq = max(0, min(p.N, p.len_k[b]));
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;

@@ -274,9 +274,14 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
 
 
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
-            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True):
+            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
+    if seq_lens is not None:
+        if pattern != L.PATTERN_LOCAL:
+            raise ValueError("seq_lens is supported by the local pattern only")
+        if seq_lens.dtype != torch.int32 or seq_lens.shape != (B,) or seq_lens.device != q.device or not seq_lens.is_contiguous():
+            raise ValueError("seq_lens must be a contiguous int32 tensor of shape (B,) on the device of q")
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("sparse self-attention needs q, k, v of one shape")
     q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
@@ -298,6 +303,8 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     a.dtype, a.B, a.H, a.L, a.D = _dtype_code(q), B, H, Lq, D
     a.pattern, a.block_len, a.aux = pattern, int(block_len), int(aux)
     a.sm_scale = float(sm_scale)
+    if seq_lens is not None:
+        a.seq_lens = seq_lens.data_ptr()
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
     lib = L.load()
     ws_bytes = lib.t5a_sparse_workspace_bytes(pattern, B, H, Lq, D, int(block_len), int(aux))
@@ -310,12 +317,16 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     return o
 
 
-def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128):
+def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128,
+                                     seq_lens=None):
     """Sliding-window self-attention: key j visible to query i iff |j-i| < block_len, bias bucket(j-i).
 
     The op of T5LocalAttention (src/turbot5/model/attentions.py:583-638) without
-    blocking, K/V triplication or a bias tensor.  q,k,v (B,H,L,D)."""
-    return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE)
+    blocking, K/V triplication or a bias tensor.  q,k,v (B,H,L,D).
+    ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; keys past a sequence's length are
+    not attended (the mask of src/turbot5/model/utils.py:174-188 for its valid query rows)."""
+    return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE,
+                   seq_lens=seq_lens)
 
 
 def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
