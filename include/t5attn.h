@@ -81,7 +81,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 105
+#define T5A_ABI_VERSION 106
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -172,10 +172,13 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           reference computes them, attentions.py:722-732, :807-814).
  *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
  *           (B,H,n_side,D) projected block aggregates, bias bucket(g - min(i/aux, n_side-1)).
- * seq_lens (optional, LOCAL only): (B) int32 on the device, the number of valid tokens of each
+ * seq_lens (optional, LOCAL and TGLOBAL): (B) int32 on the device, the number of valid tokens of each
  * right-padded sequence.  Keys at or past a sequence's length are not attended (the key half of the
  * reference's local mask, src/turbot5/model/utils.py:174-188); rows past the length are still
  * written (from the keys left in their window, zeros when there are none) and mean nothing.
+ * TGLOBAL: a sequence of length n has n / aux side tokens, its tokens past the last full block
+ * counting into the last one (utils.py:191-237 for a right-padded mask); side_k/side_v rows past
+ * them are not read.
  * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
  * the G global rows, which attend all L keys, are computed as key splits spread over the whole
  * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
@@ -231,6 +234,9 @@ int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
  * weight's type when that is 16 bit, else fp32 (torch type promotion of the reference code).
  * Arithmetic as the reference's eager path: fp32 variance and scaling, the scaled value rounded to
  * a 16-bit weight's type before the product; block sums are rounded to the input type first.
+ * seq_lens (optional, group > 1 only): (batches) int32 on the device, valid rows of each right-padded
+ * batch element: it has seq_len / group groups (its rows past the last full group join that group,
+ * padding rows are left out); output rows past them are zero.
  * residual (optional, group == 1 only): rows of x's type and shape with row stride
  * residual_row_stride; the kernel normalises x + residual (rounded to x's type, as torch's add leaves
  * it) and also writes that sum to sum_out (x's type, rows contiguous like y, 16-byte aligned; must
@@ -244,6 +250,7 @@ typedef struct t5a_rmsnorm_args {
     int32_t x_dtype; int32_t weight_dtype; float eps;
     int32_t reserved;
     const void* residual; void* sum_out; int64_t residual_row_stride;
+    const int32_t* seq_lens;
 } t5a_rmsnorm_args;
 int t5a_rmsnorm(const t5a_rmsnorm_args* args, t5a_stream_t stream);
 

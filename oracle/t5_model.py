@@ -61,29 +61,32 @@ def basic_self_attention(sd: SD, prefix: str, cfg, hidden: torch.Tensor, table: 
         out = O.block_attention_blocked(q, k, v, table, cfg.sliding_window, cfg.global_block_size, None, nb, md)
     elif attention_type == "transient-global":
         gbs = cfg.global_block_size
-        side = tglobal_side_inputs(hidden, gbs, sd[prefix + "global_input_layer_norm.weight"], cfg.layer_norm_epsilon)
+        side = tglobal_side_inputs(hidden, gbs, sd[prefix + "global_input_layer_norm.weight"], cfg.layer_norm_epsilon,
+                                   key_mask)
         sk = _heads(side @ sd[prefix + "k.weight"].T, H, D)
         sv = _heads(side @ sd[prefix + "v.weight"].T, H, D)
-        out = tglobal_attention(q, k, v, sk, sv, table, cfg.sliding_window, gbs, nb, md)
+        out = tglobal_attention(q, k, v, sk, sv, table, cfg.sliding_window, gbs, nb, md, key_mask)
     else:
         raise KeyError(attention_type)
     return _merge(out) @ sd[prefix + "o.weight"].T
 
 
-def tglobal_side_inputs(hidden, gbs, norm_weight, eps):
+def tglobal_side_inputs(hidden, gbs, norm_weight, eps, attention_mask=None):
     """Block sums (trailing tokens join the last full block, utils.py:206-212) -> RMSNorm."""
     B, L, _ = hidden.shape
-    block_ids, seg = O.make_global_fixed_block_ids(torch.ones(B, L), gbs)
+    block_ids, seg = O.make_global_fixed_block_ids(torch.ones(B, L) if attention_mask is None else attention_mask, gbs)
     agg = O.create_global_aggregates(hidden, block_ids, seg.shape[-1])
     return O.rms_norm(agg, norm_weight, eps)
 
 
-def tglobal_attention(q, k, v, sk, sv, table, Bl, gbs, nb, md):
+def tglobal_attention(q, k, v, sk, sv, table, Bl, gbs, nb, md, attention_mask=None):
     """Blocked oracle when the reference's blocking applies, dense closed form otherwise
     (L not a multiple of the block length breaks the reference's reshape, attentions.py:575-576)."""
     B, H, L, D = q.shape
     if L % Bl == 0 or L < Bl:
-        return O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs, None, nb, md)
+        return O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs, attention_mask, nb, md)
+    if attention_mask is not None:
+        raise NotImplementedError("padding mask with a length that the reference's blocking cannot take")
     i = torch.arange(L)[:, None]
     j = torch.arange(L)[None, :]
     local = table[O.relative_position_bucket(j - i, True, nb, md)].permute(2, 0, 1).unsqueeze(0)

@@ -63,12 +63,12 @@ def test_attention_module_output_tuple(gpu_device):
         assert out2[0].shape == (2, 96, 128)
     mask = torch.ones(2, 96, device=gpu_device)
     mask[1, 50:] = 0
-    for name in ("block", "transient-global"):       # right padding is the local pattern's only
+    with pytest.raises(NotImplementedError):         # right padding: local and transient-global only
+        T5ATTENTION_TYPES["block"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
+    mask[0, :3] = 0
+    for name in ("local", "transient-global"):       # left padding
         with pytest.raises(NotImplementedError):
             T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
-    mask[0, :3] = 0
-    with pytest.raises(NotImplementedError):         # left padding
-        T5ATTENTION_TYPES["local"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
 
 
 def test_flash_encoder_with_padding(gpu_device):
@@ -291,3 +291,19 @@ def test_local_encoder_with_right_padding(gpu_device):
     left[1, :10] = 0
     with pytest.raises(NotImplementedError), torch.no_grad():
         m(ids.to(gpu_device), left.to(gpu_device))
+
+
+def test_transient_global_encoder_with_right_padding(gpu_device):
+    """T5TransientGlobalAttention takes right-padded batches: per-sequence key limit and side-token count
+    in the kernels, the side-token producer leaves the padding out."""
+    cfg, m, sd = make(dict(SMALL, attention_type="transient-global", sliding_window=64, global_block_size=8))
+    ids = torch.randint(0, 200, (3, 256), generator=torch.Generator().manual_seed(10))
+    mask = torch.ones(3, 256)
+    mask[0, 203:] = 0                # orphan tokens after the last full side block
+    mask[2, 30:] = 0
+    want = OM.encoder_forward(sd, cfg, ids, mask, attention_type="transient-global")
+    m = m.to(gpu_device)
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
+    valid = mask.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 2e-3

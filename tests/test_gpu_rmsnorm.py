@@ -122,3 +122,27 @@ def test_layer_norm_add_norm_and_stack_equivalence(gpu_device):
             h, _, bias = blk(h, position_bias=bias)
         want = m.encoder.final_layer_norm(h)
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("L,gbs,lens", [(512, 16, [512, 300, 17, 0]), (100, 16, [99, 16, 15, 64]), (64, 8, [64, 63, 9, 1])])
+def test_side_token_producer_with_sequence_lengths(gpu_device, dtype, L, gbs, lens):
+    """Right-padded batch: a sequence of n tokens has n // gbs side tokens (its last tokens join the last
+    full block, padding is left out), the remaining output rows are zero -- the oracle's mask path."""
+    from turbot5_amd.ops import rms_norm
+    B, d = len(lens), 256
+    g = torch.Generator().manual_seed(L * 13 + gbs)
+    hidden = torch.randn(B, L, d, generator=g).to(DT[dtype])
+    w = (1.0 + 0.1 * torch.randn(d, generator=g)).to(DT[dtype])
+    mask = (torch.arange(L)[None, :] < torch.tensor(lens)[:, None]).float()
+    want = tglobal_side_inputs(hidden, gbs, w, 1e-6, mask)
+    got = rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=gbs,
+                   seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu_device))
+    assert got.shape == want.shape == (B, L // gbs, d)
+    tol = 1e-5 if dtype == "f32" else 2e-2
+    assert (got.float().cpu() - want.float()).abs().max().item() <= tol * max(1.0, want.float().abs().max().item())
+    for b, n in enumerate(lens):
+        assert (got[b, n // gbs:] == 0).all()
+    with pytest.raises(ValueError):
+        rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=1,
+                 seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu_device))

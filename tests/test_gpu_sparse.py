@@ -155,7 +155,7 @@ def test_local_with_sequence_lengths(gpu_device, dtype, L, Bl, lens):
     assert torch.equal(a, b_)
 
 
-def test_sequence_lengths_are_for_the_local_pattern_only(gpu_device):
+def test_sequence_lengths_are_not_for_the_block_pattern(gpu_device):
     from turbot5_amd import ops
     q = torch.zeros(1, 1, 128, 64, device=gpu_device, dtype=torch.bfloat16)
     lens = torch.tensor([100], dtype=torch.int32, device=gpu_device)
@@ -163,3 +163,25 @@ def test_sequence_lengths_are_for_the_local_pattern_only(gpu_device):
         ops._sparse(ops.L.PATTERN_BLOCK, q, q, q, None, 64, 16, seq_lens=lens)
     with pytest.raises(ValueError):
         ops.local_attention_with_fusing_bias(q, q, q, None, 64, seq_lens=lens.long())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,gbs,lens", [(512, 128, 16, [512, 300, 17, 129]), (256, 32, 8, [255, 7, 0, 64]),
+                                           (1024, 128, 16, [1000, 1024, 130, 15])])
+def test_tglobal_with_sequence_lengths(gpu_device, dtype, L, Bl, gbs, lens):
+    """Right-padded batch through the transient-global pattern: valid rows equal the oracle's mask path
+    (local mask, block ids with orphan tokens, side-token validity; utils.py:174-237)."""
+    from turbot5_amd.ops import transient_global_attention_with_fusing_bias
+    B, H, D = len(lens), 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=80 + i, dtype=dtype) for i in range(3))
+    sk, sv = (rnd(B, H, L // gbs, D, seed=83 + i, dtype=dtype) for i in range(2))
+    table = rnd(32, H, seed=85, scale=1.0)
+    mask = (torch.arange(L)[None, :] < torch.tensor(lens)[:, None]).float()
+    out = transient_global_attention_with_fusing_bias(*(t.to(gpu_device) for t in (q, k, v, sk, sv)),
+                                                      table.to(gpu_device), Bl, gbs,
+                                                      seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu_device))
+    want = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs, mask)
+    assert torch.isfinite(out).all()
+    for b, n in enumerate(lens):
+        if n:
+            assert (out.float().cpu()[b, :, :n] - want[b, :, :n]).abs().max().item() <= TOL[dtype], (b, n)

@@ -165,6 +165,53 @@ def test_tglobal_against_huggingface(hf, L, Bl, gbs):
     assert torch.allclose(got, want, atol=3e-5)
 
 
+@pytest.mark.parametrize("L,Bl,gbs", [(64, 16, 4), (96, 32, 8)])
+def test_tglobal_with_padding_against_huggingface(hf, L, Bl, gbs):
+    """Right-padded batch: the oracle's mask path (block ids, side-token validity, orphan tokens) against
+    LongT5TransientGlobalAttention with the same mask, on the valid query rows."""
+    B, H, D = 3, 2, 8
+    mod = hf.LongT5TransientGlobalAttention(_hf_cfg(hf, H, D, Bl, gbs), has_relative_attention_bias=True).eval()
+    table = rnd(32, H, seed=34, scale=1.0)
+    am = torch.ones(B, L)
+    am[0, L - gbs - 3:] = 0          # orphan tokens after the last full block
+    am[1, Bl + 1:] = 0
+    with torch.no_grad():
+        mod.relative_attention_bias.weight.copy_(table)
+        mod.global_relative_attention_bias.weight.copy_(table)
+        mod.global_input_layer_norm.weight.copy_(1.0 + rnd(H * D, seed=35, scale=0.1))
+        mod.o.weight.copy_(torch.eye(H * D))
+        x = rnd(B, L, H * D, seed=36, scale=1.0)
+        want = mod(x, mask=am)[0]
+        q = mod.q(x).view(B, L, H, D).transpose(1, 2)
+        k = mod.k(x).view(B, L, H, D).transpose(1, 2)
+        v = mod.v(x).view(B, L, H, D).transpose(1, 2)
+        side = O.tglobal_side_inputs(x, am, gbs, mod.global_input_layer_norm.weight, 1e-6)
+        sk = mod.k(side).view(B, -1, H, D).transpose(1, 2)
+        sv = mod.v(side).view(B, -1, H, D).transpose(1, 2)
+    got = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs, am).transpose(1, 2).reshape(B, L, H * D)
+    valid = am.bool()
+    assert torch.allclose(got[valid], want[valid], atol=3e-5)
+
+
+def test_tglobal_with_padding_equals_the_sequence_alone():
+    """A right-padded sequence of n valid tokens (n a multiple of the block length) gives, on its valid rows,
+    what the same n tokens give as an unpadded batch: side tokens n // gbs, keys up to n."""
+    H, D, L, Bl, gbs, n = 2, 4, 64, 16, 4, 32
+    q, k, v = (rnd(1, H, L, D, seed=37 + i) for i in range(3))
+    hidden = rnd(1, L, 6, seed=40, scale=1.0)
+    w = 1.0 + rnd(6, seed=41, scale=0.1)
+    proj = rnd(6, H * D, seed=42)
+    table = rnd(32, H, seed=43, scale=1.0)
+    am = (torch.arange(L)[None, :] < n).float()
+    def side(h, m):
+        s_ = O.tglobal_side_inputs(h, m, gbs, w) @ proj
+        return s_.view(1, -1, H, D).transpose(1, 2)
+    got = O.tglobal_attention_blocked(q, k, v, side(hidden, am), side(hidden, am), table, Bl, gbs, am)
+    want = O.tglobal_attention_blocked(q[:, :, :n], k[:, :, :n], v[:, :, :n], side(hidden[:, :n], None),
+                                       side(hidden[:, :n], None), table, Bl, gbs)
+    assert (got[:, :, :n] - want).abs().max().item() < 2e-6
+
+
 @pytest.mark.parametrize("L,Bl,gbs", [(48, 16, 4), (64, 8, 16), (256, 32, 1)])
 def test_tglobal_against_closed_form(L, Bl, gbs):
     H, D = 2, 4

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 105   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 106   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
@@ -80,7 +80,8 @@ class T5ARmsNormArgs(C.Structure):
                 ("batches", C.c_int64), ("rows_per_batch", C.c_int32), ("dim", C.c_int32), ("group", C.c_int32),
                 ("x_dtype", C.c_int32), ("weight_dtype", C.c_int32), ("eps", C.c_float),
                 ("reserved", C.c_int32),
-                ("residual", C.c_void_p), ("sum_out", C.c_void_p), ("residual_row_stride", C.c_int64)]
+                ("residual", C.c_void_p), ("sum_out", C.c_void_p), ("residual_row_stride", C.c_int64),
+                ("seq_lens", C.c_void_p)]
 
 
 _lib = None

@@ -42,13 +42,13 @@ class T5LayerNorm(nn.Module):
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(dim))
 
-    def forward(self, x: torch.Tensor, group: int = 1) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, group: int = 1, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """On a ROCm device: the fused HIP kernel (the reference switches to its Triton kernel there,
         modules.py:61-66).  Host tensors take the reference's eager formula (modules.py:51-59).
         ``group`` > 1 norms the sums of ``group`` consecutive rows of each sequence (side tokens)."""
         if x.is_cuda:
             from .ops import rms_norm
-            return rms_norm(x, self.weight, self.eps, group)
+            return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens)
         if group > 1:
             B, L, d = x.shape
             n = L // group
@@ -405,30 +405,33 @@ class T5TransientGlobalAttention(_SparseBase):
             self.global_relative_attention_bias = nn.Embedding(self.relative_attention_num_buckets, self.n_heads)
         self.global_input_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
-    def side_inputs(self, hidden_states: torch.Tensor) -> torch.Tensor:
+    def side_inputs(self, hidden_states: torch.Tensor, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Normalised block sums, (B, L // global_block_size, d_model); trailing tokens that do not fill
-        a block join the last one (utils.py:206-212, :249-258; attentions.py:959-966)."""
+        a block join the last one (utils.py:206-212, :249-258; attentions.py:959-966).  With ``seq_lens``
+        each right-padded sequence counts its valid tokens only."""
         B, L, d = hidden_states.shape
         gbs = self.global_block_size
         n_side = L // gbs
         if n_side == 0:
             return hidden_states.new_zeros(B, 0, d)
-        return self.global_input_layer_norm(hidden_states, group=gbs)   # block sums and norm in one kernel
+        return self.global_input_layer_norm(hidden_states, group=gbs, seq_lens=seq_lens)   # block sums and norm in one kernel
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
-        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        # right-padded batches: per-sequence key limit and side-token count in the kernels (utils.py:174-237)
+        seq_lens = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
+                                    right_padding_ok=True)
         batch_size = hidden_states.shape[0]
         adt = self._attn_dtype(hidden_states)
         q, k, v = self._qkv(hidden_states)
-        side = self.side_inputs(hidden_states)
+        side = self.side_inputs(hidden_states, seq_lens)
         side_k = self._shape(self.k(side), batch_size).to(adt)
         side_v = self._shape(self.v(side), batch_size).to(adt)
         table = self._table(position_bias)
         block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.transient_global_attention_with_fusing_bias(
             q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
-            self.relative_attention_num_buckets, self.relative_attention_max_distance)
+            self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens)
         return self._finish(out, hidden_states, table)
 
 

@@ -403,7 +403,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.sv_sb = a->side_v_strides[0]; p.sv_sh = a->side_v_strides[1]; p.sv_sr = a->side_v_strides[2];
     p.B = a->B; p.H = a->H; p.M = a->L; p.N = a->L;
     if (a->seq_lens != nullptr) {
-        if (a->pattern != T5A_PATTERN_LOCAL) return fail(T5A_ERR_PATTERN, "seq_lens is supported by the local pattern only");
+        if (a->pattern == T5A_PATTERN_BLOCK) return fail(T5A_ERR_PATTERN, "seq_lens is supported by the local and transient-global patterns only");
         p.len_k = a->seq_lens;
     }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
@@ -529,6 +529,10 @@ int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
     memset(&p, 0, sizeof(p));
     p.x = a->x; p.weight = a->weight; p.y = a->y;
     p.residual = a->residual; p.sum_out = a->residual ? a->sum_out : nullptr; p.residual_row_stride = a->residual_row_stride;
+    if (a->seq_lens != nullptr) {
+        if (a->group == 1) return fail(T5A_ERR_SHAPE, "seq_lens needs group > 1");
+        p.lens = a->seq_lens;
+    }
     p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;
     p.out_per_batch = out_per_batch;
     p.out_rows = a->batches * out_per_batch;

@@ -309,6 +309,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     }
 
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
+    int n_side = p.n_side;   // side tokens of this item's sequence (transient-global)
     int64_t q_off, k_off, v_off, o_off, lse_off;
     if (MODE == kPacked) {
         int qs = 0, ks = 0;
@@ -356,9 +357,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         h = (int)(bh - (unsigned)b * (unsigned)p.H);
         Mseq = p.M;
         Nseq = p.N;
-        // local pattern on a right-padded batch: the keys of a sequence end at its length; positions are
-        // the row indices, so nothing else changes (rows past the length see what is left of their window)
-        if (MODE == kLocal && p.len_k != nullptr) Nseq = max(0, min(p.N, p.len_k[b]));
+        // windowed patterns on a right-padded batch: the keys of a sequence end at its length; positions are
+        // the row indices, so nothing else changes (rows past the length see what is left of their window).
+        // Its side tokens are the full blocks of that length, the rest of its tokens joining the last one.
+        if ((MODE == kLocal || MODE == kTGlobal) && p.len_k != nullptr) {
+            Nseq = max(0, min(p.N, p.len_k[b]));
+            if (MODE == kTGlobal) n_side = min(p.n_side, Nseq / p.aux);
+        }
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -417,7 +422,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             seg_k[1] = reinterpret_cast<const T*>(p.side_k) + (int64_t)b * p.sk_sb + (int64_t)h * p.sk_sh;
             seg_v[1] = reinterpret_cast<const T*>(p.side_v) + (int64_t)b * p.sv_sb + (int64_t)h * p.sv_sh;
             seg_ksr[1] = (int)p.sk_sr * ES; seg_vsr[1] = (int)p.sv_sr * ES;
-            seg_end[1] = p.n_side; seg_lend[1] = p.n_side; seg_kind[1] = 2;
+            seg_end[1] = n_side; seg_lend[1] = n_side; seg_kind[1] = 2;
         }
     } else {  // kBlock
         nseg = 2;
@@ -806,7 +811,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         int qlo, qhi;
         if (kind == 0) { qlo = iw0 + P; qhi = iw1 + P; }
         else if (kind == 1) { qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
-        else { qlo = min(iw0 / p.aux, p.n_side - 1); qhi = min(iw1 / p.aux, p.n_side - 1); }
+        else { qlo = min(iw0 / p.aux, n_side - 1); qhi = min(iw1 / p.aux, n_side - 1); }
         const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
         c.skip = iw0 >= row_end;                              // wavefront without live rows
         if (CAUSAL) c.skip = c.skip || rel_min > 0;           // every key is in the future of every row
@@ -844,7 +849,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
         if (kind == 0) return ir + P;
         if (kind == 1) return ir % p.block_len + p.aux;
-        return min(ir / p.aux, p.n_side - 1);   // trailing tokens past the last full block join it
+        return min(ir / p.aux, n_side - 1);   // trailing tokens past the last full block join it
     };
 
     // K fragments of one tile (16-bit types): issued early so that the LDS latency hides behind

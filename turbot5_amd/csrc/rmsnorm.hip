@@ -46,13 +46,24 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     const int64_t b = row / p.out_per_batch;
     const int g = (int)(row - b * p.out_per_batch);
     const int first = g * p.group;
-    const int count = g == p.out_per_batch - 1 ? p.rows_per_batch - first : p.group;
+    // with per-sequence lengths a sequence has len / group groups, the rest of its rows joining the last
+    // one; output rows past them are zero
+    const int rows_b = p.lens ? max(0, min(p.rows_per_batch, p.lens[b])) : p.rows_per_batch;
+    const int groups_b = p.lens ? rows_b / p.group : p.out_per_batch;
+    const int count = g == groups_b - 1 ? rows_b - first : p.group;
     const TX* x = reinterpret_cast<const TX*>(p.x) + b * p.x_batch_stride + (int64_t)first * p.x_row_stride;
     const TX* res = p.residual ? reinterpret_cast<const TX*>(p.residual) + row * p.residual_row_stride : nullptr;
     TX* sum = res ? reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride : nullptr;
     const TW* w = reinterpret_cast<const TW*>(p.weight);
     TY* y = reinterpret_cast<TY*>(p.y) + row * p.y_row_stride;
     const int nch = p.dim / VEC;
+    if (g >= groups_b) {
+        Vec<TY, VEC> zero;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) zero.v[i] = Cvt<TY>::down(0.f);
+        for (int c = lane; c < nch; c += 64) *reinterpret_cast<Vec<TY, VEC>*>(y + c * VEC) = zero;
+        return;
+    }
 
     // chunk c of the row to normalise, as the input type holds it: the input row, or the sum of `count`
     // rows, or input + residual -- each sum rounded to the input type, as the torch expression leaves it

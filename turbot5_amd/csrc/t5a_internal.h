@@ -106,6 +106,7 @@ hipError_t launch_varlen_plan(const PlanParams& p, hipStream_t stream);
 struct RmsParams {
     const void* x; const void* weight; void* y;
     const void* residual; void* sum_out;                  // optional: normalise x + residual, write the sum (input type)
+    const int* lens;                                      // optional (group > 1): valid rows per batch element
     int64_t residual_row_stride;
     int64_t x_batch_stride, x_row_stride, y_row_stride;   // elements
     int64_t out_rows;        // batches * out_per_batch

@@ -278,8 +278,8 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
     if seq_lens is not None:
-        if pattern != L.PATTERN_LOCAL:
-            raise ValueError("seq_lens is supported by the local pattern only")
+        if pattern == L.PATTERN_BLOCK:
+            raise ValueError("seq_lens is supported by the local and transient-global patterns only")
         if seq_lens.dtype != torch.int32 or seq_lens.shape != (B,) or seq_lens.device != q.device or not seq_lens.is_contiguous():
             raise ValueError("seq_lens must be a contiguous int32 tensor of shape (B,) on the device of q")
     if k.shape != q.shape or v.shape != q.shape:
@@ -341,15 +341,17 @@ def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scal
 
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
-                                                sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128):
+                                                sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128, seq_lens=None):
     """Sliding window plus side tokens, the op of T5TransientGlobalAttention
-    (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D)."""
+    (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D).
+    ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; a sequence of n tokens has
+    n // global_block_size side tokens (src/turbot5/model/utils.py:191-237) and its keys end at n."""
     return _sparse(L.PATTERN_TGLOBAL, q, k, v, bias, block_len, global_block_size, side_k, side_v, sm_scale,
-                   NUM_BUCKETS, MAX_DISTANCE)
+                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1,
-             residual: Optional[torch.Tensor] = None):
+             residual: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None):
     """T5 RMS norm over the last dimension (src/turbot5/model/modules.py:51-59).
 
     With ``residual`` (same shape and dtype as x, group 1) the kernel normalises ``x + residual`` and
@@ -359,6 +361,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     ``group`` > 1: x is (B, L, d) and row r of the (B, L // group, d) result is the norm of the sum of
     rows [r*group, (r+1)*group) of its sequence, trailing rows joining the last group: the side-token
     producer of transient-global attention (src/turbot5/model/utils.py:249-258, :206-212).
+    ``seq_lens`` (B,) int32 with ``group`` > 1: valid rows of each right-padded sequence; a sequence of n rows
+    has n // group groups (rows past the last full one join it), output rows past them are zero.
     The result has the weight's dtype when that is 16 bit, else fp32, as torch promotes the reference code."""
     if not (x.is_cuda and weight.is_cuda):
         raise RuntimeError("x and weight must be on a ROCm device: this path has no CPU implementation")
@@ -395,6 +399,11 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     a.x_strides = (C.c_int64 * 2)(*strides)
     a.batches, a.rows_per_batch, a.dim, a.group = batches, rows, d, int(group)
     a.x_dtype, a.weight_dtype, a.eps = _dtype_code(x2), _dtype_code(w), float(eps)
+    if seq_lens is not None:
+        if group == 1 or seq_lens.dtype != torch.int32 or seq_lens.shape != (batches,) or seq_lens.device != x.device \
+                or not seq_lens.is_contiguous():
+            raise ValueError("seq_lens needs group > 1 and a contiguous int32 tensor of shape (B,) on the device of x")
+        a.seq_lens = seq_lens.data_ptr()
     total = None
     if r2 is not None:
         total = torch.empty(x.shape, dtype=x.dtype, device=x.device)
