@@ -221,3 +221,29 @@ def test_mask_info_is_not_inherited_by_another_tensor():
     del m
     gc.collect()
     assert ref() is None
+
+
+def test_sequence_length_arguments_are_checked_without_gpu(lib):
+    """seq_lens belongs to the windowed patterns and to the grouped norm; the checks come before any launch"""
+    handle = lib.load()
+    s = lib.T5ASparseArgs()
+    s.dtype, s.B, s.H, s.L, s.D, s.pattern, s.block_len, s.aux = 0, 1, 1, 256, 64, 2, 64, 16    # block pattern
+    s.q = s.k = s.v = s.o = 0x1000
+    for name in ("q_strides", "k_strides", "v_strides", "o_strides"):
+        setattr(s, name, (C.c_int64 * 3)(256 * 64, 256 * 64, 64))
+    s.seq_lens = 0x3000
+    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7
+    assert b"seq_lens" in handle.t5a_last_error()
+    r = lib.T5ARmsNormArgs()
+    r.x, r.weight, r.y = 0x1000, 0x2000, 0x4000
+    r.x_strides = (C.c_int64 * 2)(0, 64)
+    r.batches, r.rows_per_batch, r.dim, r.group = 1, 8, 64, 1
+    r.x_dtype, r.weight_dtype, r.eps = 0, 0, 1e-6
+    r.seq_lens = 0x3000
+    assert handle.t5a_rmsnorm(C.byref(r), None) == -4
+    assert b"seq_lens" in handle.t5a_last_error()
+    r.seq_lens = None
+    r.residual, r.sum_out, r.residual_row_stride, r.group, r.rows_per_batch = 0x5000, 0x6000, 64, 2, 8
+    assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # a residual needs group == 1
+    r.group, r.sum_out = 1, 0x1000
+    assert handle.t5a_rmsnorm(C.byref(r), None) == -5          # sum_out must not be x
