@@ -202,6 +202,24 @@ def extra_workloads(torch, dev, steps, full):
             dt = time.perf_counter() - t0
         out["greedy_decode_B64_mem8192"] = {"steps": steps_dec, "ms_per_step": round(dt / steps_dec * 1e3, 3),
                                             "tokens_per_s": round(64 * steps_dec / dt, 1)}
+        # small batches are bound by host launches: the same loop against one HIP graph per step
+        # (whole calls timed: cross-attention K/V projection of the memory + 64 steps)
+        with torch.no_grad():
+            for bsz in (8, 1):
+                memb = mem[:bsz].contiguous()
+                res = {}
+                for name, fn in (("eager", lambda: model.greedy_decode(encoder_outputs=memb, max_new_tokens=steps_dec)),
+                                 ("graphed", lambda: model.greedy_decode_graphed(memb, steps_dec))):
+                    fn()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    fn()
+                    torch.cuda.synchronize()
+                    res[name] = time.perf_counter() - t0
+                out[f"greedy_decode_B{bsz}_mem8192"] = {
+                    "steps": steps_dec, "eager_ms_per_step": round(res["eager"] / steps_dec * 1e3, 3),
+                    "graphed_ms_per_step": round(res["graphed"] / steps_dec * 1e3, 3),
+                    "graphed_tokens_per_s": round(bsz * steps_dec / res["graphed"], 1)}
         # the split-K cross-attention alone: one layer-step reads K and V of the whole memory once
         g = torch.Generator().manual_seed(7)
         kc = (0.5 * torch.randn(64, 8192, 12, 64, generator=g)).to(torch.bfloat16).to(dev).transpose(1, 2)

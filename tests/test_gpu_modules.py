@@ -307,3 +307,29 @@ def test_transient_global_encoder_with_right_padding(gpu_device):
         got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
     valid = mask.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("attention_dtype", [None, torch.bfloat16])
+def test_graphed_greedy_decode_equals_eager(gpu_device, attention_dtype):
+    """One HIP graph per decoding step (static KV cache, key length read from device memory).  The graph is
+    captured once and replayed for every step of every later call: three memories, eager decoding and
+    synchronisations in between, every call checked against the eager loop (tokens, and logits to rounding)."""
+    from turbot5_amd import T5Config, T5Model
+    torch.manual_seed(0)
+    cfg = T5Config(**dict(SMALL, attention_type="flash", attention_dtype=attention_dtype))
+    m = T5Model(cfg).eval().to(gpu_device)
+    steps = 10
+    for trial in range(3):
+        mem = torch.randn(3, 600, 128, generator=torch.Generator().manual_seed(trial)).to(gpu_device)
+        want = m.greedy_decode(encoder_outputs=mem, max_new_tokens=steps)
+        torch.cuda.synchronize()
+        got, logits = m.greedy_decode_graphed(mem, steps, return_logits=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
+        # logits of the eager pass over the same tokens (teacher forcing through the full decoder)
+        dec_in = torch.cat([torch.full((3, 1), cfg.decoder_start_token_id, device=gpu_device), want[:, :-1]], dim=1)
+        with torch.no_grad():
+            ref = m(None, dec_in, encoder_outputs=mem)[0]
+        tol = 2e-3 if attention_dtype is None else 6e-2
+        assert (logits - ref.float()).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
+    assert len(m._decode_graphs) == 1          # one capture served all three calls

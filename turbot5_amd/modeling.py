@@ -318,3 +318,99 @@ class T5Model(nn.Module):
             tokens = logits[:, -1].argmax(dim=-1, keepdim=True)
             out.append(tokens)
         return torch.cat(out, dim=1)
+
+    @torch.no_grad()
+    def greedy_decode_graphed(self, encoder_outputs: torch.Tensor, max_new_tokens: int = 16,
+                              return_logits: bool = False):
+        """Greedy decoding with one HIP graph per decoding step instead of a few hundred launches.
+
+        The step has fixed shapes: the self-attention keys and values live in preallocated
+        (B, max_new_tokens, H, D) caches that the step appends to at a position held in device memory, and
+        the packed kernel reads the current key length of every sequence from device memory too
+        (``seq_lens_k``); cross-attention keys and values are projected once, outside the graph, and read
+        by the split-K kernel.  The graph and its buffers are kept per (batch, memory length, step count)
+        and reused by later calls.  Same tokens as ``greedy_decode`` up to rounding in the logits (the
+        self-attention runs through the packed instead of the dense entry point).  All-ones encoder mask only.
+        """
+        from . import ops
+        dec, cfg = self.decoder, self.config
+        B, N, d = encoder_outputs.shape
+        dev = encoder_outputs.device
+        first = dec.block[0].layer[0].SelfAttention
+        H, D = first.n_heads, first.key_value_proj_dim
+        adt = first._attn_dtype(encoder_outputs)
+        key = (B, N, int(max_new_tokens), str(dev), encoder_outputs.dtype, adt, bool(return_logits))
+        cache = self.__dict__.setdefault("_decode_graphs", {})
+        st = cache.get(key)
+        if st is None:
+            T = int(max_new_tokens)
+            st = cache[key] = dict(
+                tok=torch.zeros(B, 1, dtype=torch.long, device=dev), pos=torch.zeros(1, dtype=torch.long, device=dev),
+                lens=torch.ones(B, dtype=torch.int32, device=dev), out=torch.zeros(B, T, dtype=torch.long, device=dev),
+                kc=[torch.zeros(B, T, H, D, dtype=adt, device=dev) for _ in dec.block],
+                vc=[torch.zeros(B, T, H, D, dtype=adt, device=dev) for _ in dec.block],
+                ck=[torch.empty(B, N, H, D, dtype=adt, device=dev) for _ in dec.block],
+                cv=[torch.empty(B, N, H, D, dtype=adt, device=dev) for _ in dec.block],
+                cu_q=torch.arange(B + 1, dtype=torch.int32, device=dev),
+                cu_k=torch.arange(B + 1, dtype=torch.int32, device=dev) * T,
+                logits=torch.zeros(B, T, cfg.vocab_size, device=dev) if return_logits else None, graph=None)
+        T = st["out"].shape[1]
+        table = first.relative_attention_bias.weight
+        nb, md = first.relative_attention_num_buckets, first.relative_attention_max_distance
+        scale = cfg.d_model ** -0.5
+
+        def step():
+            tok, pos, lens = st["tok"], st["pos"], st["lens"]
+            hidden, pending = dec.embed_tokens(tok), None
+            for l, blk in enumerate(dec.block):
+                sa, ca, ff = blk.layer[0], blk.layer[1], blk.layer[2]
+                attn, cross = sa.SelfAttention, ca.EncDecAttention
+                hidden, normed = sa.layer_norm.add_norm(hidden, pending)
+                q = attn.q(normed).view(B, H, D).to(adt)
+                st["kc"][l].index_copy_(1, pos, attn.k(normed).view(B, 1, H, D).to(adt))
+                st["vc"][l].index_copy_(1, pos, attn.v(normed).view(B, 1, H, D).to(adt))
+                o = ops.flash_attention_with_fusing_bias_varlen(
+                    q, st["kc"][l].view(B * T, H, D), st["vc"][l].view(B * T, H, D), table, st["cu_q"], st["cu_k"],
+                    1, T, causal=True, sm_scale=1.0, NUM_BUCKETS=nb, MAX_DISTANCE=md, seq_lens_k=lens,
+                    launch_plan=False)
+                pending = attn.o(o.reshape(B, 1, H * D).to(hidden.dtype))
+                hidden, normed = ca.layer_norm.add_norm(hidden, pending)
+                q = cross._shape(cross.q(normed), B).to(adt)
+                o = ops.flash_decoding_attention(q, st["ck"][l].transpose(1, 2), st["cv"][l].transpose(1, 2), None, 1.0)
+                pending = cross.o(cross._unshape(o, B).to(hidden.dtype))
+                hidden, pending = ff.step(hidden, pending)
+            hidden = dec.final_layer_norm.add_norm(hidden, pending)[1]
+            logits = self.lm_head(hidden * scale)[:, -1]
+            if st["logits"] is not None:
+                st["logits"].index_copy_(1, pos, logits.float().unsqueeze(1))
+            nxt = logits.argmax(dim=-1, keepdim=True)
+            st["out"].index_copy_(1, pos, nxt)
+            tok.copy_(nxt)
+            pos.add_(1)
+            lens.add_(1)
+
+        def reset():
+            st["tok"].fill_(cfg.decoder_start_token_id)
+            st["pos"].zero_()
+            st["lens"].fill_(1)
+
+        for l, blk in enumerate(dec.block):      # cross-attention keys and values of this memory, once
+            cross = blk.layer[1].EncDecAttention
+            st["ck"][l].copy_(cross.k(encoder_outputs).view(B, N, H, D))
+            st["cv"][l].copy_(cross.v(encoder_outputs).view(B, N, H, D))
+        if st["graph"] is None:
+            reset()
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):        # warm-up outside the capture: library handles, allocator
+                step()
+            torch.cuda.current_stream(dev).wait_stream(side)
+            reset()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            st["graph"] = graph
+        reset()
+        for _ in range(T):
+            st["graph"].replay()
+        return (st["out"].clone(), st["logits"].clone()) if return_logits else st["out"].clone()
