@@ -333,3 +333,11 @@ def test_graphed_greedy_decode_equals_eager(gpu_device, attention_dtype):
         tol = 2e-3 if attention_dtype is None else 6e-2
         assert (logits - ref.float()).abs().max().item() <= tol * max(1.0, ref.abs().max().item())
     assert len(m._decode_graphs) == 1          # one capture served all three calls
+    graph = next(iter(m._decode_graphs.values()))["graph"]
+    m.to(torch.float32 if attention_dtype is None else torch.float32)      # same dtype: parameters stay where they are
+    m.greedy_decode_graphed(mem, steps)
+    assert next(iter(m._decode_graphs.values()))["graph"] is graph
+    m.lm_head.weight = torch.nn.Parameter(m.lm_head.weight.detach().clone())   # a parameter that moved: capture again
+    got = m.greedy_decode_graphed(mem, steps)
+    assert next(iter(m._decode_graphs.values()))["graph"] is not graph
+    assert torch.equal(got, m.greedy_decode(encoder_outputs=mem, max_new_tokens=steps))

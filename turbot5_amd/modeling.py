@@ -340,7 +340,13 @@ class T5Model(nn.Module):
         H, D = first.n_heads, first.key_value_proj_dim
         adt = first._attn_dtype(encoder_outputs)
         key = (B, N, int(max_new_tokens), str(dev), encoder_outputs.dtype, adt, bool(return_logits))
+        # a graph holds the addresses of the weights it was captured with: parameters that moved since
+        # (``.to(...)``, a new ``nn.Parameter``) invalidate every captured step; values copied in place do not
+        weights = tuple(p.data_ptr() for p in self.decoder.parameters()) + (self.lm_head.weight.data_ptr(),)
         cache = self.__dict__.setdefault("_decode_graphs", {})
+        if self.__dict__.get("_decode_graph_weights") != weights:
+            cache.clear()
+            self.__dict__["_decode_graph_weights"] = weights
         st = cache.get(key)
         if st is None:
             T = int(max_new_tokens)
