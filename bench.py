@@ -180,6 +180,22 @@ def extra_workloads(torch, dev, steps, full):
                                                    "attention_tflops_lower_bound": round(attn_flops / ms / 1e9, 1)}
     del enc
     if full:
+        # ---- the baseline's small configuration (T5-small, 4 x 512 ids): a pass is a hundred short launches, bound by
+        # the host; the same pass as one HIP graph
+        from turbot5_amd import GraphedForward
+        small = dict(vocab_size=32128, d_model=512, d_kv=64, d_ff=2048, num_layers=6, num_heads=8, dropout_rate=0.0,
+                     attention_type="flash")
+        torch.manual_seed(0)
+        for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            sm = T5EncoderModel(T5Config(**small)).eval().to(dev).to(dt)
+            ids = torch.randint(0, 32128, (4, 512), generator=torch.Generator().manual_seed(0)).to(dev)
+            graphed = GraphedForward(sm, ids)
+            with torch.no_grad():
+                _, ms_e = time_kernel(torch, lambda: sm(ids), 50, 10)
+            _, ms_g = time_kernel(torch, lambda: graphed(ids), 50, 10)
+            out[f"t5_small_encoder_B4_L512_{tag}"] = {"eager_ms": round(ms_e, 3), "graphed_ms": round(ms_g, 3),
+                                                      "graphed_tokens_per_s": round(2048 / (ms_g * 1e-3), 1)}
+            del sm, graphed
         # ---- greedy decoding, batch 64 over an 8192-token encoder memory, 64 steps
         torch.manual_seed(0)
         model = T5Model(T5Config(attention_dtype=torch.bfloat16, **base)).eval().to(dev)

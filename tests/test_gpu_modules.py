@@ -341,3 +341,27 @@ def test_graphed_greedy_decode_equals_eager(gpu_device, attention_dtype):
     got = m.greedy_decode_graphed(mem, steps)
     assert next(iter(m._decode_graphs.values()))["graph"] is not graph
     assert torch.equal(got, m.greedy_decode(encoder_outputs=mem, max_new_tokens=steps))
+
+
+@pytest.mark.parametrize("attention_type,extra", [("flash", {}), ("local", dict(sliding_window=64)),
+                                                  ("transient-global", dict(sliding_window=64, global_block_size=8))])
+def test_encoder_forward_as_one_graph(gpu_device, attention_type, extra):
+    """A fixed-shape encoder pass captured once and replayed: several inputs, eager passes and
+    synchronisations in between, every replay checked against the eager result."""
+    from turbot5_amd import GraphedForward
+    cfg, m, sd = make(dict(SMALL, attention_type=attention_type, **extra))
+    m = m.to(gpu_device)
+    ids = torch.randint(0, 200, (2, 256), generator=torch.Generator().manual_seed(11)).to(gpu_device)
+    graphed = GraphedForward(m, ids)
+    for trial in range(4):
+        ids = torch.randint(0, 200, (2, 256), generator=torch.Generator().manual_seed(20 + trial)).to(gpu_device)
+        with torch.no_grad():
+            want = m(ids)
+        torch.cuda.synchronize()
+        got = graphed(ids)
+        torch.cuda.synchronize()
+        assert (got - want).abs().max().item() <= 1e-5, trial
+    with pytest.raises(ValueError):
+        graphed(ids[:, :100])
+    with pytest.raises(ValueError):
+        graphed(ids, None)

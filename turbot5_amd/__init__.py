@@ -17,3 +17,4 @@ from .attentions import (  # noqa: F401
     T5TransientGlobalAttention,
 )
 from .modeling import T5EncoderModel, T5Model, T5Stack  # noqa: F401
+from .graphs import GraphedForward  # noqa: F401
