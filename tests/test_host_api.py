@@ -247,3 +247,26 @@ def test_sequence_length_arguments_are_checked_without_gpu(lib):
     assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # a residual needs group == 1
     r.group, r.sum_out = 1, 0x1000
     assert handle.t5a_rmsnorm(C.byref(r), None) == -5          # sum_out must not be x
+
+
+def test_packed_batch_layout_and_mask_kinds():
+    """Host logic either side of the packed kernel: which masks run in place, which are right padded (the
+    windowed patterns' case), and the packed layout a whole stack runs on."""
+    from turbot5_amd import attentions as A
+    A._MASK_INFO.clear()
+    ones = torch.ones(2, 5)
+    assert A._mask_info(ones) == (True, None) and A.packed_batch(ones) is None
+    right = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1], [0, 0, 0, 0, 0]])
+    all_ones, (kind, (lens, cu), extra) = A._mask_info(right)
+    assert not all_ones and kind == "lens" and extra["right_padded"]
+    assert lens.tolist() == [3, 5, 0] and cu.tolist() == [0, 5, 10, 15]
+    pb = A.packed_batch(right)
+    assert pb.indices.tolist() == [0, 1, 2, 5, 6, 7, 8, 9] and pb.cu_seqlens.tolist() == [0, 3, 8, 8]
+    assert (pb.batch, pb.length, pb.max_len) == (3, 5, 5) and A.packed_batch(right) is pb
+    left = torch.tensor([[0, 0, 1, 1, 1], [1, 1, 1, 1, 0]])
+    _, (kind, (lens, cu), extra) = A._mask_info(left)
+    assert kind == "lens" and not extra["right_padded"] and lens.tolist() == [3, 4] and cu.tolist() == [2, 5, 10]
+    holes = torch.tensor([[1, 0, 1, 1, 0], [1, 1, 1, 1, 1]])
+    _, (kind, (indices, cu, max_len), _) = A._mask_info(holes)
+    assert kind == "packed" and indices.tolist() == [0, 2, 3, 5, 6, 7, 8, 9] and cu.tolist() == [0, 3, 8]
+    assert A.packed_batch(holes).indices is indices
