@@ -329,7 +329,8 @@ class T5Model(nn.Module):
         the packed kernel reads the current key length of every sequence from device memory too
         (``seq_lens_k``); cross-attention keys and values are projected once, outside the graph, and read
         by the split-K kernel.  The graph and its buffers are kept per (batch, memory length, step count)
-        and reused by later calls.  Same tokens as ``greedy_decode`` up to rounding in the logits (the
+        and reused by later calls (the two most recent shapes; ``model._decode_graphs.clear()`` frees them).
+        Same tokens as ``greedy_decode`` up to rounding in the logits (the
         self-attention runs through the packed instead of the dense entry point).  All-ones encoder mask only.
         """
         from . import ops
@@ -349,6 +350,8 @@ class T5Model(nn.Module):
             self.__dict__["_decode_graph_weights"] = weights
         st = cache.get(key)
         if st is None:
+            while len(cache) >= 2:      # each entry owns the K/V buffers of its batch: keep the two latest shapes
+                cache.pop(next(iter(cache)))
             T = int(max_new_tokens)
             st = cache[key] = dict(
                 tok=torch.zeros(B, 1, dtype=torch.long, device=dev), pos=torch.zeros(1, dtype=torch.long, device=dev),
