@@ -356,8 +356,10 @@ class T5Model(nn.Module):
             st = cache[key] = dict(
                 tok=torch.zeros(B, 1, dtype=torch.long, device=dev), pos=torch.zeros(1, dtype=torch.long, device=dev),
                 lens=torch.ones(B, dtype=torch.int32, device=dev), out=torch.zeros(B, T, dtype=torch.long, device=dev),
-                kc=[torch.zeros(B, T, H, D, dtype=adt, device=dev) for _ in dec.block],
-                vc=[torch.zeros(B, T, H, D, dtype=adt, device=dev) for _ in dec.block],
+                # self-attention cache: keys and values of a position side by side, so one copy appends both
+                kv=[torch.zeros(B, T, 2, H, D, dtype=adt, device=dev) for _ in dec.block],
+                # q, k and v projections of the self-attention as one GEMM: a copy of the three weights
+                wqkv=[torch.empty(3 * H * D, cfg.d_model, dtype=first.q.weight.dtype, device=dev) for _ in dec.block],
                 ck=[torch.empty(B, N, H, D, dtype=adt, device=dev) for _ in dec.block],
                 cv=[torch.empty(B, N, H, D, dtype=adt, device=dev) for _ in dec.block],
                 cu_q=torch.arange(B + 1, dtype=torch.int32, device=dev),
@@ -375,11 +377,12 @@ class T5Model(nn.Module):
                 sa, ca, ff = blk.layer[0], blk.layer[1], blk.layer[2]
                 attn, cross = sa.SelfAttention, ca.EncDecAttention
                 hidden, normed = sa.layer_norm.add_norm(hidden, pending)
-                q = attn.q(normed).view(B, H, D).to(adt)
-                st["kc"][l].index_copy_(1, pos, attn.k(normed).view(B, 1, H, D).to(adt))
-                st["vc"][l].index_copy_(1, pos, attn.v(normed).view(B, 1, H, D).to(adt))
+                qkv = nn.functional.linear(normed, st["wqkv"][l]).view(B, 3, H, D).to(adt)
+                kv = st["kv"][l]
+                kv.index_copy_(1, pos, qkv[:, 1:].unsqueeze(1))
+                rows = kv.view(B * T, 2, H, D)
                 o = ops.flash_attention_with_fusing_bias_varlen(
-                    q, st["kc"][l].view(B * T, H, D), st["vc"][l].view(B * T, H, D), table, st["cu_q"], st["cu_k"],
+                    qkv[:, 0], rows[:, 0], rows[:, 1], table, st["cu_q"], st["cu_k"],
                     1, T, causal=True, sm_scale=1.0, NUM_BUCKETS=nb, MAX_DISTANCE=md, seq_lens_k=lens,
                     launch_plan=False)
                 pending = attn.o(o.reshape(B, 1, H * D).to(hidden.dtype))
@@ -404,6 +407,8 @@ class T5Model(nn.Module):
             st["lens"].fill_(1)
 
         for l, blk in enumerate(dec.block):      # cross-attention keys and values of this memory, once
+            attn = blk.layer[0].SelfAttention
+            torch.cat([attn.q.weight, attn.k.weight, attn.v.weight], dim=0, out=st["wqkv"][l])   # current values
             cross = blk.layer[1].EncDecAttention
             st["ck"][l].copy_(cross.k(encoder_outputs).view(B, N, H, D))
             st["cv"][l].copy_(cross.v(encoder_outputs).view(B, N, H, D))
