@@ -365,3 +365,27 @@ def test_encoder_forward_as_one_graph(gpu_device, attention_type, extra):
         graphed(ids[:, :100])
     with pytest.raises(ValueError):
         graphed(ids, None)
+
+
+def test_graphed_greedy_decode_over_padded_memories(gpu_device):
+    """Encoder memories of different lengths: the captured step reads each memory's first row and length
+    from device buffers, so one graph serves masks of the same shape with other lengths."""
+    from turbot5_amd import T5Config, T5Model
+    torch.manual_seed(1)
+    m = T5Model(T5Config(**dict(SMALL, attention_type="flash"))).eval().to(gpu_device)
+    steps = 8
+    for trial, lens in enumerate(([600, 17, 333], [5, 600, 128], [600, 600, 599])):
+        mem = torch.randn(3, 600, 128, generator=torch.Generator().manual_seed(30 + trial)).to(gpu_device)
+        mask = (torch.arange(600)[None, :] < torch.tensor(lens)[:, None]).float().to(gpu_device)
+        if trial == 1:
+            mask = mask.flip(1)          # left padding
+        want = m.greedy_decode(encoder_outputs=mem, attention_mask=mask, max_new_tokens=steps)
+        torch.cuda.synchronize()
+        got = m.greedy_decode_graphed(mem, steps, attention_mask=mask)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
+    assert len(m._decode_graphs) == 1
+    holes = torch.ones(3, 600, device=gpu_device)
+    holes[0, 10:20] = 0
+    with pytest.raises(NotImplementedError):
+        m.greedy_decode_graphed(mem, steps, attention_mask=holes)

@@ -321,7 +321,7 @@ class T5Model(nn.Module):
 
     @torch.no_grad()
     def greedy_decode_graphed(self, encoder_outputs: torch.Tensor, max_new_tokens: int = 16,
-                              return_logits: bool = False):
+                              return_logits: bool = False, attention_mask: Optional[torch.Tensor] = None):
         """Greedy decoding with one HIP graph per decoding step instead of a few hundred launches.
 
         The step has fixed shapes: the self-attention keys and values live in preallocated
@@ -331,8 +331,19 @@ class T5Model(nn.Module):
         by the split-K kernel.  The graph and its buffers are kept per (batch, memory length, step count)
         and reused by later calls (the two most recent shapes; ``model._decode_graphs.clear()`` frees them).
         Same tokens as ``greedy_decode`` up to rounding in the logits (the
-        self-attention runs through the packed instead of the dense entry point).  All-ones encoder mask only.
+        self-attention runs through the packed instead of the dense entry point).
+        ``attention_mask``: the encoder's (B, N) mask.  Memories padded on either side are read in place by the
+        packed kernel, with the first row and the length of every memory in device buffers of the graph (so
+        later calls may bring other lengths); masks with holes are not taken here.
         """
+        from .attentions import _mask_info
+        mem_rows = None
+        if attention_mask is not None:
+            all_ones, unpad = _mask_info(attention_mask)
+            if not all_ones:
+                if unpad[0] != "lens":
+                    raise NotImplementedError("greedy_decode_graphed takes encoder masks without holes; use greedy_decode")
+                mem_rows = unpad[1]          # (lengths, first rows in the (B*N) layout)
         from . import ops
         dec, cfg = self.decoder, self.config
         B, N, d = encoder_outputs.shape
@@ -340,7 +351,7 @@ class T5Model(nn.Module):
         first = dec.block[0].layer[0].SelfAttention
         H, D = first.n_heads, first.key_value_proj_dim
         adt = first._attn_dtype(encoder_outputs)
-        key = (B, N, int(max_new_tokens), str(dev), encoder_outputs.dtype, adt, bool(return_logits))
+        key = (B, N, int(max_new_tokens), str(dev), encoder_outputs.dtype, adt, bool(return_logits), mem_rows is not None)
         # a graph holds the addresses of the weights it was captured with: parameters that moved since
         # (``.to(...)``, a new ``nn.Parameter``) invalidate every captured step; values copied in place do not
         weights = tuple(p.data_ptr() for p in self.decoder.parameters()) + (self.lm_head.weight.data_ptr(),)
@@ -364,6 +375,8 @@ class T5Model(nn.Module):
                 cv=[torch.empty(B, N, H, D, dtype=adt, device=dev) for _ in dec.block],
                 cu_q=torch.arange(B + 1, dtype=torch.int32, device=dev),
                 cu_k=torch.arange(B + 1, dtype=torch.int32, device=dev) * T,
+                mem_lens=torch.zeros(B, dtype=torch.int32, device=dev),
+                mem_cu=torch.zeros(B + 1, dtype=torch.int32, device=dev),
                 logits=torch.zeros(B, T, cfg.vocab_size, device=dev) if return_logits else None, graph=None)
         T = st["out"].shape[1]
         table = first.relative_attention_bias.weight
@@ -387,9 +400,16 @@ class T5Model(nn.Module):
                     launch_plan=False)
                 pending = attn.o(o.reshape(B, 1, H * D).to(hidden.dtype))
                 hidden, normed = ca.layer_norm.add_norm(hidden, pending)
-                q = cross._shape(cross.q(normed), B).to(adt)
-                o = ops.flash_decoding_attention(q, st["ck"][l].transpose(1, 2), st["cv"][l].transpose(1, 2), None, 1.0)
-                pending = cross.o(cross._unshape(o, B).to(hidden.dtype))
+                if mem_rows is None:
+                    q = cross._shape(cross.q(normed), B).to(adt)
+                    o = ops.flash_decoding_attention(q, st["ck"][l].transpose(1, 2), st["cv"][l].transpose(1, 2), None, 1.0)
+                    pending = cross.o(cross._unshape(o, B).to(hidden.dtype))
+                else:
+                    o = ops.flash_attention_with_fusing_bias_varlen(
+                        cross.q(normed).view(B, H, D).to(adt), st["ck"][l].view(B * N, H, D), st["cv"][l].view(B * N, H, D),
+                        None, st["cu_q"], st["mem_cu"], 1, N, causal=False, sm_scale=1.0, seq_lens_k=st["mem_lens"],
+                        launch_plan=False)
+                    pending = cross.o(o.reshape(B, 1, H * D).to(hidden.dtype))
                 hidden, pending = ff.step(hidden, pending)
             hidden = dec.final_layer_norm.add_norm(hidden, pending)[1]
             logits = self.lm_head(hidden * scale)[:, -1]
@@ -406,6 +426,9 @@ class T5Model(nn.Module):
             st["pos"].zero_()
             st["lens"].fill_(1)
 
+        if mem_rows is not None:
+            st["mem_lens"].copy_(mem_rows[0])
+            st["mem_cu"].copy_(mem_rows[1])
         for l, blk in enumerate(dec.block):      # cross-attention keys and values of this memory, once
             attn = blk.layer[0].SelfAttention
             torch.cat([attn.q.weight, attn.k.weight, attn.v.weight], dim=0, out=st["wqkv"][l])   # current values
