@@ -81,7 +81,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 106
+#define T5A_ABI_VERSION 107
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -218,6 +218,11 @@ typedef struct t5a_splitk_args {
     int64_t bias_strides[4];
     int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
     int32_t num_splits; float sm_scale;
+    /* optional, (B) int32 on the device: batch element b only has the keys [key_starts[b],
+     * key_starts[b] + key_lens[b]) of its N rows (a padded encoder memory; key_starts NULL = 0).  The
+     * reference masks such keys with an additive bias in T5Attention (src/turbot5/model/attentions.py:235-236);
+     * its split-K kernel has no counterpart. */
+    const int32_t* key_lens; const int32_t* key_starts;
 } t5a_splitk_args;
 int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, int32_t num_splits);
 int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);

@@ -185,3 +185,33 @@ def test_tglobal_with_sequence_lengths(gpu_device, dtype, L, Bl, gbs, lens):
     for b, n in enumerate(lens):
         if n:
             assert (out.float().cpu()[b, :, :n] - want[b, :, :n]).abs().max().item() <= TOL[dtype], (b, n)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,S", [(1, 1000, 4), (1, 8192, None), (3, 500, 7)])
+def test_splitk_over_padded_memories(gpu_device, dtype, M, N, S):
+    """Each batch element only has the keys [start, start + len) of its N rows: equal to dense attention over
+    exactly those keys; an element without keys comes out zero; splits that hold no valid key drop out."""
+    from turbot5_amd.ops import flash_decoding_attention
+    B, H, D = 5, 3, 64
+    q = rnd(B, H, M, D, seed=90, dtype=dtype)
+    k, v = (rnd(B, H, N, D, seed=91 + i, dtype=dtype) for i in range(2))
+    lens = [N, N // 3, 1, 0, N - 7]
+    starts = [0, 5, N - 1, 0, 7]
+    dq, dk, dv = (t.to(gpu_device) for t in (q, k, v))
+    tl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    ts = torch.tensor(starts, dtype=torch.int32, device=gpu_device)
+    out = flash_decoding_attention(dq, dk, dv, None, 1.0, num_splits=S, key_lens=tl, key_starts=ts).float().cpu()
+    for b in range(B):
+        if lens[b] == 0:
+            assert (out[b] == 0).all()
+            continue
+        sl = slice(starts[b], starts[b] + lens[b])
+        want = O.basic_attention(q[b:b + 1].float(), k[b:b + 1, :, sl].float(), v[b:b + 1, :, sl].float(), None)
+        assert (out[b] - want[0]).abs().max().item() <= TOL[dtype], b
+    # right padding only: starts may be left out
+    right = flash_decoding_attention(dq, dk, dv, None, 1.0, num_splits=S, key_lens=tl).float().cpu()
+    want = O.basic_attention(q[1:2].float(), k[1:2, :, :lens[1]].float(), v[1:2, :, :lens[1]].float(), None)
+    assert (right[1] - want[0]).abs().max().item() <= TOL[dtype]
+    with pytest.raises(ValueError):
+        flash_decoding_attention(dq, dk, dv, None, 1.0, key_starts=ts)

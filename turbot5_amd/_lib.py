@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 106   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 107   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
@@ -71,7 +71,8 @@ class T5ASplitKArgs(C.Structure):
                 ("q_strides", C.c_int64 * 3), ("k_strides", C.c_int64 * 3), ("v_strides", C.c_int64 * 3),
                 ("o_strides", C.c_int64 * 3), ("bias_strides", C.c_int64 * 4),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("M", C.c_int32), ("N", C.c_int32),
-                ("D", C.c_int32), ("num_splits", C.c_int32), ("sm_scale", C.c_float)]
+                ("D", C.c_int32), ("num_splits", C.c_int32), ("sm_scale", C.c_float),
+                ("key_lens", C.c_void_p), ("key_starts", C.c_void_p)]
 
 
 class T5ARmsNormArgs(C.Structure):

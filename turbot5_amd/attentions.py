@@ -260,7 +260,18 @@ class T5FlashAttention(_T5AttentionBase):
             if key_value_states is None and seq_length == key_length:
                 plan = plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt, seq_length,
                                          ops._stream(hidden_states)), ops.LaunchPlan())   # one per stream
-            if kind == "lens":
+            if kind == "lens" and table is None and not self.causal and seq_length <= 8 and key_length >= 512:
+                # few query rows over long padded memories (incremental decoding): the split-K kernel with
+                # each memory's first key and key count
+                lens_k, cu_k = unpad
+                starts = plans.get("key_starts")
+                if starts is None:
+                    starts = plans["key_starts"] = (cu_k[:batch_size] - torch.arange(
+                        batch_size, device=dev, dtype=torch.int32) * key_length).contiguous()
+                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, 1.0,
+                                                           key_lens=lens_k, key_starts=starts)
+                kind = "done"
+            elif kind == "lens":
                 # rows padded on either side: the kernel walks the padded (B*L, H, D) layout with a start row
                 # and a length per sequence; nothing is gathered or scattered (the reference unpads and pads, attentions.py:492-511)
                 def rows(t, n):
@@ -288,7 +299,7 @@ class T5FlashAttention(_T5AttentionBase):
                 cu_q = torch.arange(0, (batch_size + 1) * seq_length, seq_length, dtype=torch.int32,
                                     device=hidden_states.device)
                 indices_q, max_q = None, seq_length
-            if kind != "lens":
+            if kind not in ("lens", "done"):
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
                     q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
                     NUM_BUCKETS=nb, MAX_DISTANCE=md, launch_plan=plan)

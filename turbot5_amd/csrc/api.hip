@@ -490,6 +490,8 @@ int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
     SplitKParams p;
     memset(&p, 0, sizeof(p));
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.bias = a->attn_bias;
+    if (a->key_starts != nullptr && a->key_lens == nullptr) return fail(T5A_ERR_NULL, "key_starts given without key_lens");
+    p.key_lens = a->key_lens; p.key_starts = a->key_starts;
     const int64_t rows = (int64_t)a->B * a->H * a->num_splits * a->M;
     p.part_o = reinterpret_cast<float*>(a->workspace);
     p.part_l = p.part_o + rows * a->D;

@@ -81,8 +81,13 @@ __global__ __launch_bounds__(SK_THREADS) void splitk_partial_kernel(const SplitK
     const int b = blockIdx.z / mblocks;
     const int m0 = (blockIdx.z - b * mblocks) * MB;
     const int per = p.N / p.S;
-    const int lo = s * per;
-    const int hi = (s == p.S - 1) ? p.N : lo + per;
+    int lo = s * per;
+    int hi = (s == p.S - 1) ? p.N : lo + per;
+    if (p.key_lens != nullptr) {   // a padded memory: the split keeps what it holds of the valid keys (maybe nothing)
+        const int first = p.key_starts != nullptr ? p.key_starts[b] : 0;
+        lo = max(lo, first);
+        hi = min(hi, first + p.key_lens[b]);
+    }
     const int tid = threadIdx.x;
     const int c = tid % LPK, slot = tid / LPK;
 

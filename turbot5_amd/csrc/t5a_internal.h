@@ -81,6 +81,7 @@ struct SplitKParams {
     int64_t b_sb, b_sh, b_sr, b_sc;
     int B, H, M, N, S;
     float sm_scale;
+    const int* key_lens; const int* key_starts;   // optional: batch element b only has the keys [start, start + len)
 };
 hipError_t launch_splitk(const SplitKParams& p, int dtype, int D, hipStream_t stream);
 // only the merge over splits (part_o, part_l, part_m -> o)

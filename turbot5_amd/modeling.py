@@ -332,9 +332,9 @@ class T5Model(nn.Module):
         and reused by later calls (the two most recent shapes; ``model._decode_graphs.clear()`` frees them).
         Same tokens as ``greedy_decode`` up to rounding in the logits (the
         self-attention runs through the packed instead of the dense entry point).
-        ``attention_mask``: the encoder's (B, N) mask.  Memories padded on either side are read in place by the
-        packed kernel, with the first row and the length of every memory in device buffers of the graph (so
-        later calls may bring other lengths); masks with holes are not taken here.
+        ``attention_mask``: the encoder's (B, N) mask.  Memories padded on either side are read by the split-K
+        kernel with the first key and the key count of every memory in device buffers of the graph (so later
+        calls may bring other lengths); masks with holes are not taken here.
         """
         from .attentions import _mask_info
         mem_rows = None
@@ -376,7 +376,7 @@ class T5Model(nn.Module):
                 cu_q=torch.arange(B + 1, dtype=torch.int32, device=dev),
                 cu_k=torch.arange(B + 1, dtype=torch.int32, device=dev) * T,
                 mem_lens=torch.zeros(B, dtype=torch.int32, device=dev),
-                mem_cu=torch.zeros(B + 1, dtype=torch.int32, device=dev),
+                mem_starts=torch.zeros(B, dtype=torch.int32, device=dev),
                 logits=torch.zeros(B, T, cfg.vocab_size, device=dev) if return_logits else None, graph=None)
         T = st["out"].shape[1]
         table = first.relative_attention_bias.weight
@@ -400,16 +400,12 @@ class T5Model(nn.Module):
                     launch_plan=False)
                 pending = attn.o(o.reshape(B, 1, H * D).to(hidden.dtype))
                 hidden, normed = ca.layer_norm.add_norm(hidden, pending)
-                if mem_rows is None:
-                    q = cross._shape(cross.q(normed), B).to(adt)
-                    o = ops.flash_decoding_attention(q, st["ck"][l].transpose(1, 2), st["cv"][l].transpose(1, 2), None, 1.0)
-                    pending = cross.o(cross._unshape(o, B).to(hidden.dtype))
-                else:
-                    o = ops.flash_attention_with_fusing_bias_varlen(
-                        cross.q(normed).view(B, H, D).to(adt), st["ck"][l].view(B * N, H, D), st["cv"][l].view(B * N, H, D),
-                        None, st["cu_q"], st["mem_cu"], 1, N, causal=False, sm_scale=1.0, seq_lens_k=st["mem_lens"],
-                        launch_plan=False)
-                    pending = cross.o(o.reshape(B, 1, H * D).to(hidden.dtype))
+                q = cross._shape(cross.q(normed), B).to(adt)
+                o = ops.flash_decoding_attention(
+                    q, st["ck"][l].transpose(1, 2), st["cv"][l].transpose(1, 2), None, 1.0,
+                    key_lens=st["mem_lens"] if mem_rows is not None else None,
+                    key_starts=st["mem_starts"] if mem_rows is not None else None)
+                pending = cross.o(cross._unshape(o, B).to(hidden.dtype))
                 hidden, pending = ff.step(hidden, pending)
             hidden = dec.final_layer_norm.add_norm(hidden, pending)[1]
             logits = self.lm_head(hidden * scale)[:, -1]
@@ -428,7 +424,7 @@ class T5Model(nn.Module):
 
         if mem_rows is not None:
             st["mem_lens"].copy_(mem_rows[0])
-            st["mem_cu"].copy_(mem_rows[1])
+            st["mem_starts"].copy_(mem_rows[1][:B] - torch.arange(B, device=dev, dtype=torch.int32) * N)
         for l, blk in enumerate(dec.block):      # cross-attention keys and values of this memory, once
             attn = blk.layer[0].SelfAttention
             torch.cat([attn.q.weight, attn.k.weight, attn.v.weight], dim=0, out=st["wqkv"][l])   # current values

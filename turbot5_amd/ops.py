@@ -449,14 +449,24 @@ def flash_attn_v2_fwd(q, k, v, bias, causal, sm_scale, NUM_SPLITS=None, BLOCK_M=
     return out, part_l, part_m
 
 
-def flash_decoding_attention(q, k, v, bias=None, sm_scale=1.0, num_splits=None) -> torch.Tensor:
-    """Split-K attention returning only the merged output in q's dtype."""
-    return _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype=q.dtype)[0]
+def flash_decoding_attention(q, k, v, bias=None, sm_scale=1.0, num_splits=None, key_lens=None,
+                             key_starts=None) -> torch.Tensor:
+    """Split-K attention returning only the merged output in q's dtype.
+
+    ``key_lens`` / ``key_starts`` (optional (B,) int32 device tensors): batch element b only has the keys
+    [start, start + len) of its N rows -- a padded encoder memory, which the reference masks with an additive
+    bias (src/turbot5/model/attentions.py:235-236).  Rows of a batch element without keys come out zero."""
+    return _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype=q.dtype, key_lens=key_lens, key_starts=key_starts)[0]
 
 
-def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype):
+def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype, key_lens=None, key_starts=None):
     _check_inputs(q, k, v)
     B, H, M, D = q.shape
+    for name, t in (("key_lens", key_lens), ("key_starts", key_starts)):
+        if t is not None and (t.dtype != torch.int32 or t.shape != (B,) or t.device != q.device or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous int32 tensor of shape (B,) on the device of q")
+    if key_starts is not None and key_lens is None:
+        raise ValueError("key_starts needs key_lens")
     N = k.shape[2]
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
@@ -477,6 +487,9 @@ def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype):
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.num_splits, a.sm_scale = S, float(sm_scale)
+    if key_lens is not None:
+        a.key_lens = key_lens.data_ptr()
+        a.key_starts = key_starts.data_ptr() if key_starts is not None else None
     with _on_device(q):
         L.check(lib.t5a_fwd_splitk(C.byref(a), _stream(q)))
     rows = B * H * S * M
