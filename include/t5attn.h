@@ -239,7 +239,7 @@ int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
  * weight's type when that is 16 bit, else fp32 (torch type promotion of the reference code).
  * Arithmetic as the reference's eager path: fp32 variance and scaling, the scaled value rounded to
  * a 16-bit weight's type before the product; block sums are rounded to the input type first.
- * seq_lens (optional, group > 1 only): (batches) int32 on the device, valid rows of each right-padded
+ * seq_lens (optional, not together with residual): (batches) int32 on the device, valid rows of each right-padded
  * batch element: it has seq_len / group groups (its rows past the last full group join that group,
  * padding rows are left out); output rows past them are zero.
  * residual (optional, group == 1 only): rows of x's type and shape with row stride

@@ -143,6 +143,11 @@ def test_side_token_producer_with_sequence_lengths(gpu_device, dtype, L, gbs, le
     assert (got.float().cpu() - want.float()).abs().max().item() <= tol * max(1.0, want.float().abs().max().item())
     for b, n in enumerate(lens):
         assert (got[b, n // gbs:] == 0).all()
+    # one side token per token (group 1): every valid row normalised by itself, padding rows zero
+    tl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    one = rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=1, seq_lens=tl)
+    want1 = tglobal_side_inputs(hidden, 1, w, 1e-6, mask)
+    assert one.shape == want1.shape == (B, L, d)
+    assert (one.float().cpu() - want1.float()).abs().max().item() <= tol * max(1.0, want1.float().abs().max().item())
     with pytest.raises(ValueError):
-        rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=1,
-                 seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu_device))
+        rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=1, seq_lens=tl, residual=hidden.to(gpu_device))

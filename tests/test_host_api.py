@@ -240,10 +240,11 @@ def test_sequence_length_arguments_are_checked_without_gpu(lib):
     r.batches, r.rows_per_batch, r.dim, r.group = 1, 8, 64, 1
     r.x_dtype, r.weight_dtype, r.eps = 0, 0, 1e-6
     r.seq_lens = 0x3000
-    assert handle.t5a_rmsnorm(C.byref(r), None) == -4
+    r.residual, r.sum_out, r.residual_row_stride = 0x5000, 0x6000, 64
+    assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # lengths and a residual do not go together
     assert b"seq_lens" in handle.t5a_last_error()
     r.seq_lens = None
-    r.residual, r.sum_out, r.residual_row_stride, r.group, r.rows_per_batch = 0x5000, 0x6000, 64, 2, 8
+    r.group, r.rows_per_batch = 2, 8
     assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # a residual needs group == 1
     r.group, r.sum_out = 1, 0x1000
     assert handle.t5a_rmsnorm(C.byref(r), None) == -5          # sum_out must not be x

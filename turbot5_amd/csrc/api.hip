@@ -532,7 +532,7 @@ int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
     p.x = a->x; p.weight = a->weight; p.y = a->y;
     p.residual = a->residual; p.sum_out = a->residual ? a->sum_out : nullptr; p.residual_row_stride = a->residual_row_stride;
     if (a->seq_lens != nullptr) {
-        if (a->group == 1) return fail(T5A_ERR_SHAPE, "seq_lens needs group > 1");
+        if (a->residual != nullptr) return fail(T5A_ERR_SHAPE, "seq_lens and residual cannot be combined");
         p.lens = a->seq_lens;
     }
     p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;

@@ -361,7 +361,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     ``group`` > 1: x is (B, L, d) and row r of the (B, L // group, d) result is the norm of the sum of
     rows [r*group, (r+1)*group) of its sequence, trailing rows joining the last group: the side-token
     producer of transient-global attention (src/turbot5/model/utils.py:249-258, :206-212).
-    ``seq_lens`` (B,) int32 with ``group`` > 1: valid rows of each right-padded sequence; a sequence of n rows
+    ``seq_lens`` (B,) int32 for x of shape (B, L, d), not together with ``residual``: valid rows of each right-padded sequence; a sequence of n rows
     has n // group groups (rows past the last full one join it), output rows past them are zero.
     The result has the weight's dtype when that is 16 bit, else fp32, as torch promotes the reference code."""
     if not (x.is_cuda and weight.is_cuda):
@@ -379,7 +379,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
         r2 = residual.detach().reshape(-1, d)
         if r2.stride(-1) != 1 or r2.stride(0) % 8 != 0 or r2.data_ptr() % 16 != 0:
             r2 = r2.contiguous()
-    if group == 1:
+    if group == 1 and seq_lens is None:
         x2 = x_.reshape(-1, d)
         if x2.stride(-1) != 1 or x2.stride(0) % 8 != 0 or x2.data_ptr() % 16 != 0:
             x2 = x2.contiguous()
@@ -400,9 +400,9 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     a.batches, a.rows_per_batch, a.dim, a.group = batches, rows, d, int(group)
     a.x_dtype, a.weight_dtype, a.eps = _dtype_code(x2), _dtype_code(w), float(eps)
     if seq_lens is not None:
-        if group == 1 or seq_lens.dtype != torch.int32 or seq_lens.shape != (batches,) or seq_lens.device != x.device \
-                or not seq_lens.is_contiguous():
-            raise ValueError("seq_lens needs group > 1 and a contiguous int32 tensor of shape (B,) on the device of x")
+        if residual is not None or seq_lens.dtype != torch.int32 or seq_lens.shape != (batches,) \
+                or seq_lens.device != x.device or not seq_lens.is_contiguous():
+            raise ValueError("seq_lens must be a contiguous int32 tensor of shape (B,) on the device of x, without residual")
         a.seq_lens = seq_lens.data_ptr()
     total = None
     if r2 is not None:
