@@ -365,6 +365,17 @@ def test_encoder_forward_as_one_graph(gpu_device, attention_type, extra):
         graphed(ids[:, :100])
     with pytest.raises(ValueError):
         graphed(ids, None)
+    if attention_type == "flash":      # a mask keeps the pattern it was captured with
+        mask = torch.ones(2, 256, device=gpu_device)
+        mask[1, 200:] = 0
+        masked = GraphedForward(m, ids, mask)
+        with torch.no_grad():
+            want = m(ids, mask)
+        assert (masked(ids, mask.clone()) - want).abs().max().item() <= 1e-5
+        other = mask.clone()
+        other[1, 150:] = 0
+        with pytest.raises(ValueError):
+            masked(ids, other)
 
 
 def test_graphed_greedy_decode_over_padded_memories(gpu_device):

@@ -7,8 +7,10 @@ the static buffers, the graph runs, the static output is returned (valid until t
 
 Only tensors may vary between calls, and only in their values: shapes, dtypes, ``None``-ness and every
 non-tensor argument are fixed at capture.  Host-side decisions of the module (is the mask all ones,
-how many tokens are valid) are taken once, at capture, from the example inputs -- so pass masks only
-when every later mask has the same pattern, or run without one.  Inference only.
+how many tokens are valid) are taken once, at capture, from the example inputs -- so a mask must keep
+the pattern it had at capture.  Arguments that look like one ((B, L) tensors that are not integer ids:
+floating, bool or int32 and smaller) are compared with the captured pattern on every call, which costs one
+host synchronisation, and a different pattern raises.  Inference only.
 """
 from __future__ import annotations
 
@@ -41,6 +43,9 @@ class GraphedForward:
         if torch.is_tensor(static):
             if not torch.is_tensor(new) or new.shape != static.shape or new.dtype != static.dtype:
                 raise ValueError(f"argument {name}: the captured graph takes a {tuple(static.shape)} {static.dtype} tensor")
+            if static.dim() == 2 and static.dtype != torch.long and not torch.equal(new != 0, static != 0):
+                raise ValueError(f"argument {name} looks like an attention mask and its pattern differs from the one "
+                                 "the graph was captured with; capture a graph for this pattern or run the module itself")
             static.copy_(new)
         elif torch.is_tensor(new) or new != static:
             raise ValueError(f"argument {name} was {static!r} at capture and cannot change")
