@@ -476,3 +476,36 @@ def test_scores_that_keep_climbing_along_the_keys(gpu_device, dtype, causal):
     assert (out.float().cpu() - want).abs().max().item() <= tol
     # the row sum adds probabilities as the matrix core sees them (rounded to the 16-bit type)
     assert (lse.cpu() - want_lse).abs().max().item() <= (2e-3 if dtype == torch.float32 else 1e-2)
+
+
+def test_raw_ctypes_binding_as_a_reference_maintainer_would_write_it(gpu_device):
+    """The binding shown to maintainers of the reference (a drop-in body for flash_attn_v2_fwd_bias,
+    fused_bias_attention.py:23-59): plain ctypes on the C ABI, no helper of the ops module."""
+    import ctypes as C
+    from turbot5_amd._lib import load, check, T5ADenseArgs, T5A_BF16
+
+    def flash_attn_v2_fwd_bias(q, k, v, bias_weights, causal, sm_scale):
+        B, H, M, D = q.shape
+        o = torch.empty_like(q)
+        lse = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
+        a = T5ADenseArgs()
+        a.q, a.k, a.v, a.o, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr()
+        for name, t in (("q_strides", q), ("k_strides", k), ("v_strides", v), ("o_strides", o)):
+            setattr(a, name, (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2)))
+        a.dtype, a.B, a.H, a.M, a.N, a.D = T5A_BF16, B, H, M, k.shape[2], D
+        a.causal, a.sm_scale = int(causal), float(sm_scale)
+        if bias_weights is not None:
+            a.bias.table, a.bias.table_dtype = bias_weights.data_ptr(), 1
+            a.bias.num_buckets, a.bias.max_distance = 32, 128
+            a.bias.stride_bucket, a.bias.stride_head = bias_weights.stride(0), bias_weights.stride(1)
+        with torch.cuda.device(q.device):
+            check(load().t5a_fwd_dense(C.byref(a), torch.cuda.current_stream().cuda_stream))
+        return o, lse
+
+    q, k, v = (rnd(2, 4, 300, 64, seed=70 + i, dtype=torch.bfloat16) for i in range(3))
+    table = rnd(32, 4, seed=73, scale=1.0)
+    for causal in (False, True):
+        o, lse = flash_attn_v2_fwd_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device), causal, 1.0)
+        want = O.dense_attention(q, k, v, table, causal, 1.0)
+        assert (o.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+        assert (lse.cpu() - O.dense_lse(q, k, table, causal, 1.0)).abs().max().item() <= 2e-2
