@@ -220,6 +220,17 @@ class T5FlashAttention(_T5AttentionBase):
                 f"past_key_value should have 2 past states: keys and values. Got { len(past_key_value)} past states")
         adt = self._attn_dtype(hidden_states)
 
+        # A padded memory (cross-attention without cached keys): its k and v projections run on the valid rows
+        # only and are scattered into zeros; the padding rows are never attended.
+        memory_rows, memory_layout = None, None
+        if (key_value_states is not None and varlen and key_value_states.is_cuda
+                and (past_key_value is None or past_key_value[0].shape[2] != key_value_states.shape[1])):
+            layout = packed_batch(mask)
+            n_rows = key_value_states.shape[0] * key_value_states.shape[1]
+            if layout is not None and 0 < layout.indices.numel() <= 0.85 * n_rows and mask.shape[1] == key_value_states.shape[1]:
+                memory_layout = layout
+                memory_rows = index_first_axis(key_value_states.reshape(n_rows, -1), layout.indices)
+
         def project(proj_layer, past):
             """keys or values: (B, H, key_length, D) in the attention dtype (attentions.py:444-469)."""
             if key_value_states is None:
@@ -228,6 +239,10 @@ class T5FlashAttention(_T5AttentionBase):
                     states = torch.cat([past, states], dim=2)
                 return states
             if past is None or past.shape[2] != key_value_states.shape[1]:
+                if memory_rows is not None:
+                    padded = pad_input(proj_layer(memory_rows).to(adt), memory_layout.indices,
+                                       memory_layout.batch, memory_layout.length)
+                    return self._shape(padded, batch_size)
                 return self._shape(proj_layer(key_value_states), batch_size).to(adt)
             return past
 

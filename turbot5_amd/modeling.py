@@ -425,12 +425,21 @@ class T5Model(nn.Module):
         if mem_rows is not None:
             st["mem_lens"].copy_(mem_rows[0])
             st["mem_starts"].copy_(mem_rows[1][:B] - torch.arange(B, device=dev, dtype=torch.int32) * N)
-        for l, blk in enumerate(dec.block):      # cross-attention keys and values of this memory, once
+        # cross-attention keys and values of this memory, once; of padded memories only the valid rows are
+        # projected (gathered once for all layers), the other rows of the buffers are never read
+        valid_rows = packed_batch(attention_mask) if mem_rows is not None else None
+        if valid_rows is not None and not 0 < valid_rows.indices.numel() <= 0.85 * B * N:
+            valid_rows = None
+        mem_valid = index_first_axis(encoder_outputs.reshape(B * N, d), valid_rows.indices) if valid_rows is not None else None
+        for l, blk in enumerate(dec.block):
             attn = blk.layer[0].SelfAttention
             torch.cat([attn.q.weight, attn.k.weight, attn.v.weight], dim=0, out=st["wqkv"][l])   # current values
             cross = blk.layer[1].EncDecAttention
-            st["ck"][l].copy_(cross.k(encoder_outputs).view(B, N, H, D))
-            st["cv"][l].copy_(cross.v(encoder_outputs).view(B, N, H, D))
+            for proj, buf in ((cross.k, st["ck"][l]), (cross.v, st["cv"][l])):
+                if mem_valid is None:
+                    buf.copy_(proj(encoder_outputs).view(B, N, H, D))
+                else:
+                    buf.view(B * N, H, D).index_copy_(0, valid_rows.indices, proj(mem_valid).view(-1, H, D).to(adt))
         if st["graph"] is None:
             reset()
             side = torch.cuda.Stream(device=dev)
