@@ -115,3 +115,27 @@ def test_tglobal_16k(gpu_device):
     for h in range(H):
         want = rows_oracle(q, kcat, vcat, table, rows, h, key_ids, rel, live)
         assert (out[0, h, rows].float() - want).abs().max().item() <= 2e-2
+
+
+def test_padded_sequences_equal_the_sequences_alone_16k(gpu_device):
+    """Size-independent property of the per-sequence lengths at L = 16384: a right-padded sequence of n
+    tokens gives, on its n rows, what the n tokens give as a batch of their own (local and transient-global
+    patterns; n a multiple of the side block so that both runs build the same side tokens)."""
+    from turbot5_amd.ops import local_attention_with_fusing_bias, transient_global_attention_with_fusing_bias
+    H, L, D, Bl, gbs = 12, 16384, 64, 128, 16
+    lens = [16384, 9600, 4112]
+    B = len(lens)
+    q, k, v = (rnd(B, H, L, D, seed=120 + i).to(gpu_device) for i in range(3))
+    sk, sv = (rnd(B, H, L // gbs, D, seed=123 + i).to(gpu_device) for i in range(2))
+    table = rnd(32, H, seed=125, scale=1.0, dtype=torch.float32).to(gpu_device)
+    tl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    loc = local_attention_with_fusing_bias(q, k, v, table, Bl, seq_lens=tl)
+    tg = transient_global_attention_with_fusing_bias(q, k, v, sk, sv, table, Bl, gbs, seq_lens=tl)
+    assert torch.isfinite(loc).all() and torch.isfinite(tg).all()
+    for b, n in enumerate(lens):
+        qa, ka, va = (t[b:b + 1, :, :n].contiguous() for t in (q, k, v))
+        alone = local_attention_with_fusing_bias(qa, ka, va, table, Bl)
+        assert (loc[b, :, :n].float() - alone[0].float()).abs().max().item() <= 2e-2, ("local", b)
+        ska, sva = (t[b:b + 1, :, :n // gbs].contiguous() for t in (sk, sv))
+        alone = transient_global_attention_with_fusing_bias(qa, ka, va, ska, sva, table, Bl, gbs)
+        assert (tg[b, :, :n].float() - alone[0].float()).abs().max().item() <= 2e-2, ("tglobal", b)
