@@ -16,10 +16,14 @@ Pinning status (what checks each function besides this file itself):
   closed form.  tests/test_oracle_sparse.py
 * ``tglobal_attention_blocked`` -- HuggingFace ``LongT5TransientGlobalAttention``
   (with its side table set equal to the local table) and the closed form.
-* ``block_attention_blocked`` -- brute-force closed form only: no third-party
-  counterpart exists and the reference holds no vectors for it, so its
-  agreement with the reference *module* is "parity unpinned"; the closed form
-  it is checked against was derived from the same reading of att.py:652-862.
+* ``block_attention_blocked`` -- vectors written from the reference's own
+  ``T5BlockAttention`` (all-ones, right-padded, left-padded and holed masks,
+  ragged last block, sequences shorter than a block; tests/golden/
+  sparse_modules.npz, made by tests/golden/make_sparse_fixtures.py in the build
+  container) and a brute-force closed form.  tests/test_oracle_fixtures.py
+* the local and transient-global functions with left padding and holes in the
+  mask -- the same fixture file (``T5LocalAttention``,
+  ``T5TransientGlobalAttention`` end to end).
 * ``splitk_merge`` -- identity with un-split dense attention.
 """
 from __future__ import annotations
