@@ -153,4 +153,7 @@ def decoder_forward(sd: SD, cfg, decoder_input_ids: torch.Tensor, memory: torch.
 
 
 def lm_logits(sd: SD, cfg, hidden: torch.Tensor) -> torch.Tensor:
-    return (hidden * (cfg.d_model ** -0.5)) @ sd["lm_head.weight"].T
+    """Tied embeddings: rescale by d_model**-0.5 before the head; untied: no rescale (modeling.py:704)."""
+    if getattr(cfg, "tie_word_embeddings", True):
+        hidden = hidden * (cfg.d_model ** -0.5)
+    return hidden @ sd["lm_head.weight"].T

@@ -33,6 +33,9 @@ class T5Config:
     pad_token_id: int = 0
     eos_token_id: int = 1
     decoder_start_token_id: int = 0
+    # T5 v1.0 ties the lm head to the input embedding and rescales the decoder output by d_model**-0.5 before
+    # it; T5 v1.1 / Flan (gated-gelu) have an untied head and no rescale (reference modeling.py:704)
+    tie_word_embeddings: bool = True
     attention_type: str = "flash"        # key of T5ATTENTION_TYPES
     sliding_window: int = 512            # block_len of local / block / transient-global
     global_block_size: int = 32          # block: number of global tokens; transient-global: tokens per side token

@@ -213,7 +213,14 @@ class T5Stack(nn.Module):
         position_bias = None
         presents: List[Optional[Tuple[torch.Tensor, ...]]] = []
         # the decoder's own padding mask has no meaning under causal attention with right padding;
-        # only the encoder mask is routed down (as key padding of self- and cross-attention)
+        # only the encoder mask is routed down (as key padding of self- and cross-attention).  Left padding
+        # or holes would change the positions the reference computes (it unpads with the mask), so they
+        # are refused rather than silently ignored.
+        if self.is_decoder and attention_mask is not None and attention_mask.is_cuda:
+            from .attentions import _mask_info
+            all_ones, unpad = _mask_info(attention_mask)
+            if not all_ones and not (unpad[0] == "lens" and unpad[2].get("right_padded")):
+                raise NotImplementedError("the decoder takes all-ones or right-padded attention masks only")
         self_mask = None if self.is_decoder else attention_mask
         packed = None
         if self.pack_padded_batches and self_mask is not None and hidden_states.is_cuda:
@@ -258,6 +265,9 @@ def _init_t5_weights(module: nn.Module, config: T5Config) -> None:
                 m.relative_attention_bias.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
                 if hasattr(m, "global_relative_attention_bias"):
                     m.global_relative_attention_bias.weight.data.normal_(mean=0.0, std=f * (d_model ** -0.5))
+    # writes through .data do not bump the version counter that the distance-LUT cache keys on
+    from . import ops
+    ops.clear_bias_luts()
 
 
 class T5EncoderModel(nn.Module):
@@ -288,6 +298,10 @@ class T5Model(nn.Module):
         self.lm_head = nn.Linear(config.d_model, config.vocab_size, bias=False)
         self.shared.weight.data.normal_(mean=0.0, std=config.initializer_factor * 1.0)
         self.lm_head.weight.data.normal_(mean=0.0, std=config.initializer_factor * 1.0)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.shared.weight
+        # tied embeddings are rescaled before the head, untied ones are not (reference modeling.py:704)
+        self.lm_scale = config.d_model ** -0.5 if config.tie_word_embeddings else 1.0
         _init_t5_weights(self, config)
 
     def forward(self, input_ids, decoder_input_ids, attention_mask=None, encoder_outputs=None,
@@ -297,8 +311,7 @@ class T5Model(nn.Module):
         hidden, presents = self.decoder(input_ids=decoder_input_ids, encoder_hidden_states=encoder_outputs,
                                         encoder_attention_mask=attention_mask, past_key_values=past_key_values,
                                         use_cache=use_cache)
-        # tied embeddings are rescaled before the head, as T5 does (t5_heads.py: sequence_output * d_model**-0.5)
-        logits = self.lm_head(hidden * (self.config.d_model ** -0.5))
+        logits = self.lm_head(hidden * self.lm_scale if self.lm_scale != 1.0 else hidden)
         return logits, encoder_outputs, presents
 
     @torch.no_grad()
@@ -381,7 +394,7 @@ class T5Model(nn.Module):
         T = st["out"].shape[1]
         table = first.relative_attention_bias.weight
         nb, md = first.relative_attention_num_buckets, first.relative_attention_max_distance
-        scale = cfg.d_model ** -0.5
+        scale = self.lm_scale
 
         def step():
             tok, pos, lens = st["tok"], st["pos"], st["lens"]

@@ -58,25 +58,43 @@ BIAS_LUT_CACHE = True
 
 
 def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int, causal: bool, ref: torch.Tensor):
+    """-> (lut buffer or None, cache key to commit after a successful launch or None)."""
     if not BIAS_LUT_CACHE or torch.cuda.is_current_stream_capturing():
-        return None   # a build recorded into a graph would not have run when the next eager launch reads it
+        return None, None   # a build recorded into a graph would not have run when the next eager launch reads it
     key = (bias.data_ptr(), bias._version, bias.stride(0), bias.stride(1), bias.dtype, H, num_buckets, max_distance,
            bool(causal), ref.device.index, _stream(ref))
     hit = _BIAS_LUTS.get(key)
+    pending = None
     if hit is None:
         nbytes = L.load().t5a_bias_lut_bytes(H, num_buckets, max_distance, int(bool(causal)))
         if nbytes <= 0:
-            return None
+            return None, None
         lut = torch.empty(nbytes, device=ref.device, dtype=torch.uint8)
-        _BIAS_LUTS[key] = (bias, lut)
-        while len(_BIAS_LUTS) > 64:
-            _BIAS_LUTS.popitem(last=False)
+        pending = key       # recorded as built only once the library has queued the build (_commit_lut)
         b.lut_ready = 0
     else:
         lut = hit[1]
         b.lut_ready = 1
     b.lut, b.lut_bytes = lut.data_ptr(), lut.numel()
-    return lut
+    return lut, pending
+
+
+def _commit_lut(keep, launched: bool):
+    """After the library call has returned without error: remember a LUT buffer that this call built.  A call
+    that returned before its launch (empty batch) or raised has not built it, and leaves no entry."""
+    if keep is None or not launched:
+        return
+    table, lut, pending, bias = keep
+    if pending is not None and lut is not None:
+        _BIAS_LUTS[pending] = (bias, lut)
+        while len(_BIAS_LUTS) > 64:
+            _BIAS_LUTS.popitem(last=False)
+
+
+def clear_bias_luts():
+    """Forget every cached distance LUT.  The cache keys on the table's identity and version counter; updates
+    that bypass the counter (``param.data.copy_``, raw kernels writing into the table) need this call."""
+    _BIAS_LUTS.clear()
 
 
 def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_distance: int, ref: torch.Tensor,
@@ -98,8 +116,9 @@ def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_dis
     b.max_distance = max_distance
     b.stride_bucket = table.stride(0)
     b.stride_head = table.stride(1)
-    lut = _bias_lut(b, bias, H, num_buckets, max_distance, causal, ref) if table.data_ptr() == bias.data_ptr() else None
-    return b, (table, lut)   # keep both alive until the launch has been queued
+    lut, pending = (_bias_lut(b, bias, H, num_buckets, max_distance, causal, ref)
+                    if table.data_ptr() == bias.data_ptr() else (None, None))
+    return b, (table, lut, pending, bias)   # alive until the launch has been queued; see _commit_lut
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -161,6 +180,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, causal)
     with _on_device(q):
         L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
+    _commit_lut(keep, B > 0 and M > 0)
     return (o, lse) if return_lse else o
 
 
@@ -185,13 +205,17 @@ class LaunchPlan:
         self.workspace = None
 
     def lookup(self, key, tensors, nbytes, device):
-        """-> (workspace, ready)"""
+        """-> (workspace, ready).  A plan that is not ready counts as built only after ``commit``."""
         if self.key == key and self.workspace is not None:
             return self.workspace, True
         if self.workspace is None or self.workspace.numel() < nbytes or self.workspace.device != device:
             self.workspace = torch.empty(nbytes, device=device, dtype=torch.uint8)
-        self.key, self.tensors = key, tensors
+        self.key, self.tensors = None, None
         return self.workspace, False
+
+    def commit(self, key, tensors):
+        """The library has queued the build for ``key`` (its call returned without error)."""
+        self.key, self.tensors = key, tensors
 
 
 def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
@@ -258,6 +282,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     wanted = launch_plan == "always" or (shared and items >= PLAN_MIN_ITEMS_SHARED) or \
         (launch_plan is True and items >= PLAN_MIN_ITEMS)
     ws_bytes = lib.t5a_varlen_workspace_bytes(B, H, total_q) if wanted else 0
+    plan_key = None
     if ws_bytes > 0:
         # under graph capture nothing runs yet: a plan recorded there must not count as built for later eager calls
         if shared and not torch.cuda.is_current_stream_capturing():
@@ -265,11 +290,17 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
             key += (B, H, D, total_q, a.dtype, a.causal, a.max_seqlen_q, a.max_seqlen_k, str(q.device))
             ws, ready = launch_plan.lookup(key, (cq, ck, lens[0], lens[1]), ws_bytes, q.device)
             a.workspace_ready = int(ready)
+            if not ready:
+                plan_key = key
         else:
             ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)   # stream-ordered reuse by torch's allocator
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
     with _on_device(q):
         L.check(lib.t5a_fwd_varlen(C.byref(a), _stream(q)))
+    launched = B > 0 and total_q > 0
+    _commit_lut(keep, launched)
+    if plan_key is not None and launched:
+        launch_plan.commit(plan_key, (cq, ck, lens[0], lens[1]))
     return (o, lse) if return_lse else o
 
 
@@ -314,6 +345,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
         a.workspace, a.workspace_bytes = workspace.data_ptr(), ws_bytes
     with _on_device(q):
         L.check(lib.t5a_fwd_sparse(C.byref(a), _stream(q)))
+    _commit_lut(keep, B > 0 and Lq > 0)
     return o
 
 
