@@ -129,7 +129,7 @@ CASES = [
     ("T5BlockAttention", 2, 40, 1, 16, 16, 8, "ones"),     # ragged last block (the reference's view() needs H == 1 for it)
     ("T5BlockAttention", 2, 10, 2, 16, 16, 4, "ones"),     # shorter than a block: full attention
     ("T5BlockAttention", 2, 48, 2, 16, 16, 16, "ones"),    # as many global tokens as a block holds
-    ("T5BlockAttention", 1, 96, 3, 8, 32, 8, "ones"),
+    ("T5BlockAttention", 1, 96, 3, 16, 32, 8, "ones"),
     ("T5BlockAttention", 2, 64, 2, 16, 16, 4, "right"),
     ("T5BlockAttention", 2, 40, 1, 16, 16, 8, "right"),
     ("T5LocalAttention", 2, 40, 1, 16, 16, 0, "right"),
@@ -144,7 +144,7 @@ CASES = [
     ("T5TransientGlobalAttention", 2, 64, 2, 16, 16, 8, "right"),
     ("T5TransientGlobalAttention", 2, 64, 2, 16, 16, 8, "left"),
     ("T5TransientGlobalAttention", 2, 64, 2, 16, 16, 8, "holes"),
-    ("T5TransientGlobalAttention", 1, 96, 3, 8, 32, 16, "right"),
+    ("T5TransientGlobalAttention", 1, 96, 3, 16, 32, 16, "right"),
 ]
 
 

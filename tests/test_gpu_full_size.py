@@ -1,5 +1,5 @@
 """Size-independent checks at the full sizes of the baseline configurations: 100k tokens dense
-(bidirectional and causal), the three sparse patterns at L = 16384.  The oracle is applied to a random
+(bidirectional and causal), the three sparse patterns at L = 16384 with 12 heads (baseline configuration 4).  The oracle is applied to a random
 subset of query rows (every key of those rows), which it finishes in seconds."""
 import pytest
 import torch
@@ -55,7 +55,7 @@ def test_dense_100k_tokens(gpu_device, causal):
 
 def test_local_16k(gpu_device):
     from turbot5_amd.ops import local_attention_with_fusing_bias
-    L, H, D, Bl = 16384, 2, 64, 128
+    L, H, D, Bl = 16384, 12, 64, 128
     q, k, v = (rnd(1, H, L, D, seed=80 + i) for i in range(3))
     table = rnd(32, H, seed=83, scale=1.0, dtype=torch.float32)
     out = local_attention_with_fusing_bias(*(t.to(gpu_device) for t in (q, k, v, table)), Bl).cpu()
@@ -72,7 +72,7 @@ def test_block_16k(gpu_device):
     """[G global tokens | own block] with rel = c - (G + r) over the list column c; block 0 loses its last
     G columns; the first G rows see every key (reference layout, attentions.py:685-691, :722-732, :788-814)."""
     from turbot5_amd.ops import block_attention_with_fusing_bias
-    L, H, D, Bl, G = 16384, 2, 64, 128, 64
+    L, H, D, Bl, G = 16384, 12, 64, 128, 64
     q, k, v = (rnd(1, H, L, D, seed=90 + i) for i in range(3))
     table = rnd(32, H, seed=93, scale=1.0, dtype=torch.float32)
     out = block_attention_with_fusing_bias(*(t.to(gpu_device) for t in (q, k, v, table)), Bl, G).cpu()
@@ -97,7 +97,7 @@ def test_block_16k(gpu_device):
 
 def test_tglobal_16k(gpu_device):
     from turbot5_amd.ops import transient_global_attention_with_fusing_bias
-    L, H, D, Bl, gbs = 16384, 2, 64, 128, 16
+    L, H, D, Bl, gbs = 16384, 12, 64, 128, 16
     Gn = L // gbs
     q, k, v = (rnd(1, H, L, D, seed=100 + i) for i in range(3))
     sk, sv = (rnd(1, H, Gn, D, seed=103 + i) for i in range(2))
