@@ -18,6 +18,16 @@
  *  - Every function returns T5A_OK (0) or a negative t5a_status; the message
  *    of the last failure on the calling thread is t5a_last_error().
  *  - Scores are q.k * sm_scale + bias; the T5 modules pass sm_scale = 1.0.
+ *  - Score precision (bf16 and fp16 inputs; the exact_scores field of the dense, varlen and sparse
+ *    arguments).  0 (default): the query rows are multiplied by sm_scale * log2(e) and rounded back to the
+ *    input type before the matrix product, a relative error of 2^-9 (bf16) on every term of a score.
+ *    With unscaled T5 scores of deviation 8 (18) the output error against fp32 math on the same inputs is
+ *    about 4.5e-2 (1.1e-1) at worst, 3.6 times below that of the reference's 'basic' path run in bf16
+ *    (src/turbot5/ops/naive_attention.py:4-23 rounds the scores themselves to bf16).  Non-zero: the query
+ *    rows enter the product as they are and the factor is applied to the fp32 result, as the reference's
+ *    fused kernel does (src/turbot5/ops/fused_bias_attention.py:323-337); the error stays near 1e-2 (the
+ *    rounding of the output) at any score magnitude and the kernels take about 11 % longer at head_dim 64.
+ *    fp32 inputs are always exact.
  *  - The relative-position bias is never materialised: kernels derive
  *    bucket(key_pos - query_pos) from integer positions and read the
  *    (num_buckets, H) table.  Bucket boundaries are computed on the host with
@@ -81,7 +91,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 107
+#define T5A_ABI_VERSION 108
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -108,6 +118,7 @@ typedef struct t5a_dense_args {
     int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
     int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
     int32_t causal; float sm_scale;
+    int32_t exact_scores; int32_t reserved;   /* exact_scores: see "Score precision" above */
     t5a_bias bias;
 } t5a_dense_args;
 int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
@@ -150,7 +161,7 @@ typedef struct t5a_varlen_args {
     int32_t dtype; int32_t B; int32_t H; int32_t D;
     int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
     int32_t causal; float sm_scale;
-    int32_t workspace_ready; int32_t reserved;
+    int32_t workspace_ready; int32_t exact_scores;
     t5a_bias bias;
 } t5a_varlen_args;
 int64_t t5a_varlen_workspace_bytes(int32_t B, int32_t H, int32_t total_q);
@@ -192,7 +203,7 @@ typedef struct t5a_sparse_args {
     int64_t side_k_strides[3]; int64_t side_v_strides[3];
     int32_t dtype; int32_t B; int32_t H; int32_t L; int32_t D;
     int32_t pattern; int32_t block_len; int32_t aux; int32_t n_side;
-    float sm_scale; int32_t reserved;
+    float sm_scale; int32_t exact_scores;
     t5a_bias bias;
     const int32_t* seq_lens;
 } t5a_sparse_args;

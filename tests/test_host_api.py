@@ -33,7 +33,7 @@ def test_header_symbols_are_exported(lib):
 def test_struct_sizes_follow_the_header(lib):
     # natural alignment, no packing: catches a field added on one side only
     assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8
-    assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 8 * 4 + C.sizeof(lib.T5ABias)
+    assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 8
     assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4 + 2 * 8
@@ -102,7 +102,9 @@ def test_workspace_sizes_and_checks_without_gpu(lib):
     # distance LUTs: (H, 4, qlen) floats with qlen = 4 * (ceil((entries + 6) / 4) ... ) as the kernel lays them out
     for causal, sat in ((0, 91), (1, 113)):           # saturation distances of 32 buckets / max_distance 128
         entries = sat + 96 + (0 if causal else sat) + 96 + 1
-        qlen = 4 * ((entries + 6) // 4 + 1)
+        quads = (entries + 6) // 4 + 1
+        quads += (4 - quads) % 16          # the four copies start 16 floats apart modulo the 64 LDS banks
+        qlen = 4 * quads
         assert handle.t5a_bias_lut_bytes(12, 32, 128, causal) == 12 * 4 * qlen * 4
     assert handle.t5a_bias_lut_bytes(12, 32, 4096, 0) == 0      # too long for the kernel's fetch: not offered
     assert handle.t5a_bias_lut_bytes(0, 32, 128, 0) == 0

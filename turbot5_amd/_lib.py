@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 107   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 108   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 
 EXPORTS = (
@@ -36,6 +36,7 @@ class T5ADenseArgs(C.Structure):
                 ("o_strides", C.c_int64 * 3),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("M", C.c_int32), ("N", C.c_int32),
                 ("D", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
+                ("exact_scores", C.c_int32), ("reserved", C.c_int32),
                 ("bias", T5ABias)]
 
 
@@ -49,7 +50,7 @@ class T5AVarlenArgs(C.Structure):
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32),
                 ("max_seqlen_k", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
-                ("workspace_ready", C.c_int32), ("reserved", C.c_int32),
+                ("workspace_ready", C.c_int32), ("exact_scores", C.c_int32),
                 ("bias", T5ABias)]
 
 
@@ -61,7 +62,7 @@ class T5ASparseArgs(C.Structure):
                 ("o_strides", C.c_int64 * 3), ("side_k_strides", C.c_int64 * 3), ("side_v_strides", C.c_int64 * 3),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("L", C.c_int32), ("D", C.c_int32),
                 ("pattern", C.c_int32), ("block_len", C.c_int32), ("aux", C.c_int32), ("n_side", C.c_int32),
-                ("sm_scale", C.c_float), ("reserved", C.c_int32),
+                ("sm_scale", C.c_float), ("exact_scores", C.c_int32),
                 ("bias", T5ABias), ("seq_lens", C.c_void_p)]
 
 

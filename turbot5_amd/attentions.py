@@ -178,6 +178,11 @@ class _T5AttentionBase(nn.Module):
     def _attn_dtype(self, x: torch.Tensor) -> torch.dtype:
         return self.config.attention_dtype or x.dtype
 
+    @property
+    def _exact(self):
+        """None (library default) or the config's choice of score precision, see ``ops.EXACT_SCORES``."""
+        return getattr(self.config, "attention_exact_scores", None)
+
     def _table(self, position_bias):
         if position_bias is None and self.has_relative_attention_bias:
             position_bias = self.relative_attention_bias.weight
@@ -259,7 +264,7 @@ class T5FlashAttention(_T5AttentionBase):
                 attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, 1.0)
             else:
                 attn_output = ops.flash_attention_with_fusing_bias(
-                    query_states, key_states, value_states, table, causal=self.causal, sm_scale=1.0,
+                    query_states, key_states, value_states, table, causal=self.causal, sm_scale=1.0, exact_scores=self._exact,
                     NUM_BUCKETS=nb, MAX_DISTANCE=md)
         else:
             if mask.shape[1] != key_length:
@@ -298,7 +303,7 @@ class T5FlashAttention(_T5AttentionBase):
                                                            dtype=torch.int32, device=dev)
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
                     rows(q_blhd, seq_length), rows(k_blhd, key_length), rows(v_blhd, key_length), table, cu_q, cu_k,
-                    seq_length, key_length, causal=self.causal, sm_scale=1.0, NUM_BUCKETS=nb, MAX_DISTANCE=md,
+                    seq_length, key_length, causal=self.causal, sm_scale=1.0, exact_scores=self._exact, NUM_BUCKETS=nb, MAX_DISTANCE=md,
                     seq_lens_q=unpad if self_attn else None, seq_lens_k=unpad,
                     launch_plan=plan)
                 attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
@@ -316,7 +321,7 @@ class T5FlashAttention(_T5AttentionBase):
                 indices_q, max_q = None, seq_length
             if kind not in ("lens", "done"):
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
-                    q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0,
+                    q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0, exact_scores=self._exact,
                     NUM_BUCKETS=nb, MAX_DISTANCE=md, launch_plan=plan)
                 if indices_q is not None:
                     attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
@@ -340,7 +345,7 @@ class T5FlashAttention(_T5AttentionBase):
                                         ops._stream(hidden_states)), ops.LaunchPlan())
         out = ops.flash_attention_with_fusing_bias_varlen(
             q, k, v, table, packed.cu_seqlens, packed.cu_seqlens, packed.max_len, packed.max_len,
-            causal=self.causal, sm_scale=1.0, NUM_BUCKETS=self.relative_attention_num_buckets,
+            causal=self.causal, sm_scale=1.0, exact_scores=self._exact, NUM_BUCKETS=self.relative_attention_num_buckets,
             MAX_DISTANCE=self.relative_attention_max_distance, launch_plan=plan)
         return (self.o(out.reshape(total, self.inner_dim).to(hidden_states.dtype)), None, table)
 
@@ -395,7 +400,8 @@ class T5LocalAttention(_SparseBase):
         block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.local_attention_with_fusing_bias(
             q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance, seq_lens=seq_lens)
+            self.relative_attention_max_distance, seq_lens=seq_lens,
+            exact_scores=self._exact)
         return self._finish(out, hidden_states, table)
 
 
@@ -414,7 +420,7 @@ class T5BlockAttention(_SparseBase):
         table = self._table(position_bias)
         out = ops.block_attention_with_fusing_bias(
             q, k, v, table, self.block_len, self.n_global_tokens, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance)
+            self.relative_attention_max_distance, exact_scores=self._exact)
         return self._finish(out, hidden_states, table)
 
 
@@ -457,7 +463,8 @@ class T5TransientGlobalAttention(_SparseBase):
         block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.transient_global_attention_with_fusing_bias(
             q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
-            self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens)
+            self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens,
+            exact_scores=self._exact)
         return self._finish(out, hidden_states, table)
 
 

@@ -44,6 +44,9 @@ class T5Config:
     # dtype the attention kernels run in; None = the dtype of the activations.  torch.bfloat16 with
     # fp32 activations gives "fp32 activations, bf16 attention".
     attention_dtype: Optional[torch.dtype] = None
+    # bf16 / fp16 attention: apply the score scale to the fp32 product instead of to the query rows (closer to
+    # fp32 math at large scores, about 11 % slower); None = the default of ``turbot5_amd.ops.EXACT_SCORES``
+    attention_exact_scores: Optional[bool] = None
     dense_act_fn: str = field(init=False, default="relu")
     is_gated_act: bool = field(init=False, default=False)
 

@@ -256,6 +256,7 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     p.total_items = (int)items;
     if (a->causal != 0 && p.tiles_per_seq > 1) causal_slices(&p, a->dtype, a->D);
     p.c1 = a->sm_scale * kLog2e;
+    p.exact_scale = a->exact_scores != 0;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
     if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
@@ -308,6 +309,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     p.tiles_per_seq = 1;
     p.align_end = 1;
     p.c1 = a->sm_scale * kLog2e;
+    p.exact_scale = a->exact_scores != 0;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
     if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     const int64_t need = t5a_varlen_workspace_bytes(a->B, a->H, a->total_q);
@@ -408,6 +410,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
     p.c1 = a->sm_scale * kLog2e;
+    p.exact_scale = a->exact_scores != 0;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;
     hipStream_t s = (hipStream_t)stream;
     if ((rc = prepare_lut(a->bias, false, s, &p))) return rc;
@@ -468,8 +471,9 @@ int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, i
     return (int64_t)B * H * num_splits * M * ((int64_t)D + 2) * (int64_t)sizeof(float);
 }
 
-int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
-    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+// The split-K forward with the workspace passed explicitly.
+static int splitk_run(const t5a_splitk_args* a, void* workspace, int64_t workspace_bytes, t5a_stream_t stream,
+                      const char* what) {
     int rc = check_common(a->dtype, a->D);
     if (rc) return rc;
     if (a->B < 0 || a->H <= 0 || a->M < 0 || a->N < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d M=%d N=%d", a->B, a->H, a->M, a->N);
@@ -484,16 +488,16 @@ int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
         if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
     }
     const int64_t need = t5a_splitk_workspace_bytes(a->B, a->H, a->M, a->D, a->num_splits);
-    if (a->workspace == nullptr || a->workspace_bytes < need)
-        return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)a->workspace_bytes);
-    if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(T5A_ERR_WORKSPACE, "%s: workspace of %lld bytes needed, %lld given", what, (long long)need, (long long)workspace_bytes);
+    if (!aligned16(workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
     SplitKParams p;
     memset(&p, 0, sizeof(p));
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.bias = a->attn_bias;
     if (a->key_starts != nullptr && a->key_lens == nullptr) return fail(T5A_ERR_NULL, "key_starts given without key_lens");
     p.key_lens = a->key_lens; p.key_starts = a->key_starts;
     const int64_t rows = (int64_t)a->B * a->H * a->num_splits * a->M;
-    p.part_o = reinterpret_cast<float*>(a->workspace);
+    p.part_o = reinterpret_cast<float*>(workspace);
     p.part_l = p.part_o + rows * a->D;
     p.part_m = p.part_l + rows;
     p.q_sb = a->q_strides[0]; p.q_sh = a->q_strides[1]; p.q_sr = a->q_strides[2];
@@ -503,7 +507,12 @@ int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
     p.b_sb = a->bias_strides[0]; p.b_sh = a->bias_strides[1]; p.b_sr = a->bias_strides[2]; p.b_sc = a->bias_strides[3];
     p.B = a->B; p.H = a->H; p.M = a->M; p.N = a->N; p.S = a->num_splits;
     p.sm_scale = a->sm_scale;
-    return finish(launch_splitk(p, a->dtype, a->D, (hipStream_t)stream), "t5a_fwd_splitk");
+    return finish(launch_splitk(p, a->dtype, a->D, (hipStream_t)stream), what);
+}
+
+int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    return splitk_run(a, a->workspace, a->workspace_bytes, stream, "t5a_fwd_splitk");
 }
 
 int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {

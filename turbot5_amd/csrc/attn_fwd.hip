@@ -13,10 +13,10 @@
 //                    (bias - running max), so the MFMA result is directly the
 //                    exp2 argument.
 //   P   = exp2(S^T)  online softmax in base 2.  The running max is only raised
-//                    when a tile exceeds it by more than 2^8 (the sums and the
-//                    output are normalised by the same stale max, so the
-//                    result is unchanged), which keeps the rescale off the
-//                    common path.
+//                    when a tile exceeds it by more than 2^24 (2^14 for fp16;
+//                    the sums and the output are normalised by the same stale
+//                    max, so the result is unchanged), which keeps the rescale
+//                    off the common path.
 //   O^T += V^T P^T   the S^T accumulators are already laid out as the B
 //                    operand (for 16-bit types after a key permutation that is
 //                    baked into the LDS layout of V^T), so P stays in registers.
@@ -114,13 +114,8 @@ constexpr int NTHREADS = 256;
 // two, so rows whose maximum creeps up over many tiles rescale their accumulators a few times, not on
 // every tile.  Probabilities then reach 2^limit: bf16 and fp32 have the exponent range for 2^24 (sums
 // and outputs are fp32 and are divided by the row sum at the end); fp16 tops out at 65504, hence 2^14.
-#ifndef T5A_RAISE
-#define T5A_RAISE 24.0f
-#endif
-template <typename T> constexpr float raise_limit() { return sizeof(T) == 2 && !__is_same(T, __bf16) ? 14.0f : T5A_RAISE; }
-#ifndef OCC
-#define OCC 2
-#endif
+template <typename T> constexpr float raise_limit() { return sizeof(T) == 2 && !__is_same(T, __bf16) ? 14.0f : 24.0f; }
+constexpr int kWorkgroupsPerCU = 2;   // 72 KB of LDS and 256 registers per lane each
 
 // table element from its bits (zero-extended for the 16-bit types)
 __device__ __forceinline__ float table_value(unsigned raw, int dtype) {
@@ -245,7 +240,7 @@ struct Geometry {
 };
 
 template <typename T, int D, int MODE, bool CAUSAL>
-__global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkgroupsPerCU) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
     using v8 = typename E::v8;
@@ -259,6 +254,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
     // head_dim 64, 16-bit types: the Q rows are staged through LDS by LDS-DMA as well (see the prologue)
     constexpr bool QDMA = G::DMA && D == 64;
+    // 16-bit inputs, two ways to apply sm_scale * log2(e).  Default: Q is pre-multiplied and rounded back to the
+    // input type, which puts a relative error of 2^-9 (bf16; 2^-12 for fp16) on every term of a score and costs
+    // nothing per tile.  exact_scale: the Q fragments stay as loaded, the accumulator input is divided by the
+    // factor and the fp32 product is multiplied by it: one more vector multiply per score (about 11 % of the
+    // run time at head_dim 64).  Wavefront-uniform, decided once per launch.
+    const bool exact = !F32 && p.exact_scale != 0;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr bool DMA = G::DMA;
@@ -580,6 +581,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     // flight.  (Q loaded into registers by the compiler would be waited for with "nothing outstanding".)
     static_assert(!QDMA || (K_TILE * ES == 8192 && V_TILE * ES == 8192 && NSK == 4 && NSV == 4 && NTHREADS == 256),
                   "the Q staging borrows 4 KB per wavefront from the last K and V ring stages");
+    // the staged Q rows are 128 bytes: rows two apart share their banks, so the 16-byte chunks are XOR-swizzled
+    // like the K tiles (on the source side of the request) and a 16-lane read phase covers all 64 banks
+    auto qswz = [](int row) { return (row >> 1) & 7; };
     const unsigned q_stage = wave < 2 ? (unsigned)(NSV * V_TILE + 3 * K_TILE) * ES + wave * 4096u
                                       : (unsigned)(3 * V_TILE) * ES + (wave - 2) * 4096u;
     if constexpr (QDMA) {
@@ -589,7 +593,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         const u32x4 rs = make_rsrc_words(qp, row_end > 0 ? (unsigned)(row_end - 1) * (unsigned)q_row_bytes + D * ES : 0u);
 #pragma unroll
         for (int r = 0; r < 4; ++r)   // 8 rows of 128 bytes per request; rows past the end arrive as zeros
-            lds_dma_16(rs, lds_base + q_stage + r * 1024, (iw0 + 8 * r + (lane >> 3)) * q_row_bytes + (lane & 7) * 16);
+            lds_dma_16(rs, lds_base + q_stage + r * 1024,
+                       (iw0 + 8 * r + (lane >> 3)) * q_row_bytes + (((lane & 7) ^ qswz(8 * r + (lane >> 3))) * 16));
     }
     if constexpr (DMA) {
         if (lut_cached) {
@@ -651,7 +656,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     if constexpr (QDMA) {
         const T* qs_rows = reinterpret_cast<const T*>(smem + q_stage);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v8*>(qs_rows + lr * D + (2 * s + hh) * 8);
+        for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const v8*>(qs_rows + lr * D + (((2 * s + hh) ^ qswz(lr)) * 8));
     }
     if constexpr (F32) {
 #pragma unroll
@@ -659,12 +664,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
             qf[2 * c] = (hh ? qraw[c][1] : qraw[c][0]) * p.c1;
             qf[2 * c + 1] = (hh ? qraw[c][3] : qraw[c][2]) * p.c1;
         }
-    } else {
+    } else if (!exact) {
 #pragma unroll
         for (int s = 0; s < KS; ++s)
 #pragma unroll
             for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)qf[s][e] * p.c1);
     }
+    // exact_scale: the accumulator input is (bias - running max) / c1 and the product is multiplied by c1
+    // afterwards; otherwise inv_c1 is 1 and the same instructions form (bias - running max) itself
+    const float inv_c1 = exact ? 1.0f / p.c1 : 1.0f;
 
     // ---------------------------------------------------------------- tile staging
     u32x4 kreg[K_PER_T];
@@ -871,6 +879,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
     auto compute_s = [&](const TileClass& c, int buf, const v8 (&ka)[NT][KS], f32x16 (&st)[NT]) {
         const int qpos = lane_qpos(c.sg);
         if (c.use_lut) {
+            const float m_neg = -m_run * inv_c1;
             const int e0 = c.j0 + 4 * hh - qpos + padl;
             const float* lb = lut + (e0 & 3) * qlen;
             const int y0 = e0 >> 2;
@@ -881,7 +890,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
                     const int y = y0 + 8 * nt + 2 * g;   // always inside the LUT, see LUT_PAD
                     const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x] - m_run;
+                    for (int x = 0; x < 4; ++x)
+                        st[nt][4 * g + x] = __builtin_fmaf(bq[x], inv_c1, m_neg);
                 }
         }
         if constexpr (F32) {
@@ -909,6 +919,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
 #pragma unroll
                     for (int s = 1; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
                 }
+            }
+            if (exact) {
+                asm volatile("");   // a real branch around the multiplies, not 32 selects
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) st[nt][r] *= p.c1;
             }
         }
     };
@@ -1044,7 +1061,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : OCC) v
         if (side != 0) side_cur = side;
         cb_cur = side_cur == 1 ? c_neg : (side_cur == 2 ? c_pos : 0.f);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) cm[r] = cb_cur - m_run;
+        for (int r = 0; r < 16; ++r) cm[r] = (cb_cur - m_run) * inv_c1;
     };
 
     // ---------------------------------------------------------------- software pipeline
@@ -1223,12 +1240,21 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
     const size_t lut_bytes = (((size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float) + 1023) & ~(size_t)1023) + 1024;
     const size_t smem = Geometry<T, D>::kTileBytes + lut_bytes;
     auto kern = fwd_kernel<T, D, MODE, CAUSAL>;
-    static std::atomic<size_t> granted{0};   // per instantiation: largest dynamic LDS size already allowed
-    if (smem > 48 * 1024 && smem > granted.load(std::memory_order_relaxed)) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    // per instantiation and device: largest dynamic LDS size already allowed (the attribute belongs to the
+    // function as loaded on one device)
+    constexpr int kMaxDevices = 64;
+    static std::atomic<size_t> granted[kMaxDevices] = {};
+    int dev = 0;
+    if (smem > 48 * 1024) {
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
-        granted.store(smem, std::memory_order_relaxed);
+        const bool known = dev >= 0 && dev < kMaxDevices;
+        if (!known || smem > granted[dev].load(std::memory_order_relaxed)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return e;
+            if (known) granted[dev].store(smem, std::memory_order_relaxed);
+        }
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
     if (MODE == kPacked && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;

@@ -16,7 +16,10 @@ constexpr int LUT_PAD = 96;
 // floats per shifted copy of the distance LUT (host and device agree through this)
 __host__ __device__ inline int lut_quads(int sat, bool causal) {
     const int entries = sat + LUT_PAD + (causal ? 0 : sat) + LUT_PAD + 1;   // rel = -sat-PAD .. (sat|0)+PAD
-    return (entries + 3 + 3) / 4 + 1;                                      // + 3 for the shifted copies
+    const int quads = (entries + 3 + 3) / 4 + 1;                           // + 3 for the shifted copies
+    // Four neighbouring lanes read the four copies at the same position: the copies start 16 floats apart
+    // modulo the 64 LDS banks (quads = 4 mod 16), so the 16 lanes of a 16-byte read phase cover all banks.
+    return quads + ((4 - quads) & 15);
 }
 
 __device__ __forceinline__ int bucket_of(const BucketSpec& s, int rel) {

@@ -49,6 +49,7 @@ struct FwdParams {
     // the kernel's tail is made of short items
     int xcd_lo[9];
     float c1;            // sm_scale * log2(e)
+    int exact_scale;     // 16-bit inputs: apply c1 to the fp32 product instead of to Q (see attn_fwd.hip)
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;
     const float* lut_global;   // optional: the distance LUTs of all heads, (H, 4, qlen) floats (lut.hip)
     int block_len, aux, n_side;

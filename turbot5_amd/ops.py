@@ -20,6 +20,17 @@ from . import _lib as L
 
 _DTYPES = {torch.bfloat16: L.T5A_BF16, torch.float32: L.T5A_F32, torch.float16: L.T5A_F16}
 
+# Score precision of the fused kernels for bf16 / fp16 inputs when a call does not say (``exact_scores=None``).
+# False: the query rows are multiplied by sm_scale * log2(e) and rounded back to the input type before the
+# matrix product (relative error 2^-9 per term in bf16; still 3.6 times more accurate than the reference's
+# 'basic' path in bf16, and within 2e-2 of fp32 math for scores of deviation up to about 4).  True: the factor
+# is applied to the fp32 product, as the reference's fused kernel does; about 11 % slower at head_dim 64.
+EXACT_SCORES = False
+
+
+def _exact(flag) -> int:
+    return int(EXACT_SCORES if flag is None else bool(flag))
+
 
 def _dtype_code(t: torch.Tensor) -> int:
     try:
@@ -152,7 +163,7 @@ def _strides3(t):
 
 
 def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                     return_lse: bool = False):
+                                     return_lse: bool = False, exact_scores: Optional[bool] = None):
     """FlashAttention forward with the T5 relative-position bias computed inside the kernel.
 
     q (B,H,M,D); k, v (B,H,N,D), any batch/head/row strides; ``bias`` is the
@@ -177,6 +188,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q_), _strides3(k_), _strides3(v_), _strides3(o)
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.exact_scores = _exact(exact_scores)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, causal)
     with _on_device(q):
         L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
@@ -221,7 +233,7 @@ class LaunchPlan:
 def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                             causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
                                             return_lse: bool = False, seq_lens_q=None, seq_lens_k=None,
-                                            launch_plan: bool = True):
+                                            launch_plan: bool = True, exact_scores: Optional[bool] = None):
     """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
 
     Positions restart at 0 in every sequence.  No host synchronisation: the
@@ -274,6 +286,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     a.total_q, a.total_k = total_q, total_k
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.exact_scores = _exact(exact_scores)
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, causal)
     lib = L.load()
     # building a plan costs about 15 us: worth it from a few thousand items on, earlier when shared
@@ -305,7 +318,7 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
 
 
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
-            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None):
+            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
     if seq_lens is not None:
@@ -334,6 +347,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     a.dtype, a.B, a.H, a.L, a.D = _dtype_code(q), B, H, Lq, D
     a.pattern, a.block_len, a.aux = pattern, int(block_len), int(aux)
     a.sm_scale = float(sm_scale)
+    a.exact_scores = _exact(exact_scores)
     if seq_lens is not None:
         a.seq_lens = seq_lens.data_ptr()
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
@@ -350,7 +364,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
 
 
 def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                     seq_lens=None):
+                                     seq_lens=None, exact_scores=None):
     """Sliding-window self-attention: key j visible to query i iff |j-i| < block_len, bias bucket(j-i).
 
     The op of T5LocalAttention (src/turbot5/model/attentions.py:583-638) without
@@ -358,28 +372,29 @@ def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM
     ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; keys past a sequence's length are
     not attended (the mask of src/turbot5/model/utils.py:174-188 for its valid query rows)."""
     return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE,
-                   seq_lens=seq_lens)
+                   seq_lens=seq_lens, exact_scores=exact_scores)
 
 
 def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
-                                     MAX_DISTANCE=128, key_splits=True):
+                                     MAX_DISTANCE=128, key_splits=True, exact_scores=None):
     """Block attention with ``n_global`` leading global tokens, the op of T5BlockAttention
     (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout.
 
     ``key_splits``: hand the library a workspace so that the global rows (which attend every key) are
     spread over the device as key splits and merged; False keeps them in one workgroup per (batch, head)."""
     return _sparse(L.PATTERN_BLOCK, q, k, v, bias, block_len, n_global, None, None, sm_scale, NUM_BUCKETS,
-                   MAX_DISTANCE, key_splits=key_splits)
+                   MAX_DISTANCE, key_splits=key_splits, exact_scores=exact_scores)
 
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
-                                                sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128, seq_lens=None):
+                                                sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128, seq_lens=None,
+                                                exact_scores=None):
     """Sliding window plus side tokens, the op of T5TransientGlobalAttention
     (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D).
     ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; a sequence of n tokens has
     n // global_block_size side tokens (src/turbot5/model/utils.py:191-237) and its keys end at n."""
     return _sparse(L.PATTERN_TGLOBAL, q, k, v, bias, block_len, global_block_size, side_k, side_v, sm_scale,
-                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens)
+                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens, exact_scores=exact_scores)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1,
