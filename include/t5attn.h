@@ -239,6 +239,21 @@ int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, i
 int t5a_fwd_splitk(const t5a_splitk_args* args, t5a_stream_t stream);
 
 /*
+ * t5a_fwd_splitk for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, kernels and
+ * results as t5a_fwd_splitk, except that args->workspace and args->workspace_bytes are ignored: the partial
+ * results go to a static device array of T5A_STATIC_SCRATCH_BYTES that is part of the library (each GPU the
+ * library runs on holds its copy until the process ends).  The call allocates and frees nothing.
+ * Limit: t5a_splitk_workspace_bytes(B, H, M, D, num_splits) <= T5A_STATIC_SCRATCH_BYTES, else
+ * T5A_ERR_WORKSPACE (batch 64, 12 heads, one query row, head_dim 64, 16 splits need 3.1 MiB).
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside a
+ * graph capture.  All calls on one GPU share the array: calls that may overlap in time (different streams,
+ * different threads) race on it; calls ordered on one stream do not.
+ */
+#define T5A_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+int t5a_fwd_splitk_static(const t5a_splitk_args* args, t5a_stream_t stream);
+
+/*
  * T5 RMS norm (no mean subtraction, no bias) and, with group > 1, the side-token producer of the
  * transient-global pattern: output row r of a sequence is the norm of the SUM of input rows
  * [r*group, (r+1)*group), the rows left over at the end of the sequence joining its last group.

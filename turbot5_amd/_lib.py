@@ -15,11 +15,13 @@ LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
 ABI_VERSION = 108   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
+STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
     "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes",
-    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_rmsnorm",
+    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
+    "t5a_rmsnorm",
 )
 
 
@@ -117,7 +119,8 @@ def load() -> C.CDLL:
         lib.t5a_bucket_lut.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32)]
         lib.t5a_bucket_lut.restype = C.c_int
         for name, typ in (("t5a_fwd_dense", T5ADenseArgs), ("t5a_fwd_varlen", T5AVarlenArgs),
-                          ("t5a_fwd_sparse", T5ASparseArgs), ("t5a_fwd_splitk", T5ASplitKArgs)):
+                          ("t5a_fwd_sparse", T5ASparseArgs), ("t5a_fwd_splitk", T5ASplitKArgs),
+                          ("t5a_fwd_splitk_static", T5ASplitKArgs)):
             fn = getattr(lib, name)
             fn.argtypes = [C.POINTER(typ), C.c_void_p]
             fn.restype = C.c_int

@@ -471,7 +471,7 @@ int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, i
     return (int64_t)B * H * num_splits * M * ((int64_t)D + 2) * (int64_t)sizeof(float);
 }
 
-// The split-K forward with the workspace passed explicitly.
+// Shared by t5a_fwd_splitk (caller's workspace) and t5a_fwd_splitk_static (the library's static scratch array).
 static int splitk_run(const t5a_splitk_args* a, void* workspace, int64_t workspace_bytes, t5a_stream_t stream,
                       const char* what) {
     int rc = check_common(a->dtype, a->D);
@@ -513,6 +513,48 @@ static int splitk_run(const t5a_splitk_args* a, void* workspace, int64_t workspa
 int t5a_fwd_splitk(const t5a_splitk_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     return splitk_run(a, a->workspace, a->workspace_bytes, stream, "t5a_fwd_splitk");
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Split-K forward for callers that cannot allocate: the partial results live in a device array that is
+// part of the library's image (every device the library runs on holds its own copy until the process ends).
+// In host code the array's name is only a handle for hipGetSymbolAddress, never a device address: the
+// address is looked up once per device, with that device current, and kept; kernels and every other use get
+// that pointer.
+static __device__ __align__(256) unsigned char scratch[T5A_STATIC_SCRATCH_BYTES];
+
+static int static_scratch(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* ptrs[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(T5A_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(T5A_ERR_LAUNCH, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> g(mu);
+    if (ptrs[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(T5A_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        ptrs[dev] = ptr;
+    }
+    *out = ptrs[dev];
+    return T5A_OK;
+}
+
+int t5a_fwd_splitk_static(const t5a_splitk_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    const int64_t need = t5a_splitk_workspace_bytes(a->B, a->H, a->M, a->D, a->num_splits);
+    if (need > (int64_t)T5A_STATIC_SCRATCH_BYTES)
+        return fail(T5A_ERR_WORKSPACE, "t5a_fwd_splitk_static: B=%d H=%d M=%d D=%d num_splits=%d need %lld bytes of partial "
+                    "results, the static scratch array holds %lld; use fewer splits or t5a_fwd_splitk with a workspace",
+                    a->B, a->H, a->M, a->D, a->num_splits, (long long)need, (long long)T5A_STATIC_SCRATCH_BYTES);
+    void* ptr = nullptr;
+    int rc = static_scratch(&ptr);
+    if (rc) return rc;
+    // nothing has to be cleared: the split kernel writes every partial row that the merge of the same call reads
+    return splitk_run(a, ptr, (int64_t)T5A_STATIC_SCRATCH_BYTES, stream, "t5a_fwd_splitk_static");
 }
 
 int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {

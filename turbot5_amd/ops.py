@@ -506,6 +506,34 @@ def flash_decoding_attention(q, k, v, bias=None, sm_scale=1.0, num_splits=None, 
     return _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype=q.dtype, key_lens=key_lens, key_starts=key_starts)[0]
 
 
+def flash_decoding_attention_static(q, k, v, out, sm_scale=1.0, num_splits=None, key_lens=None, key_starts=None):
+    """Split-K attention that allocates nothing: the caller passes the (B,H,M,D) output tensor and the partial
+    results go to the library's static scratch array (``t5a_fwd_splitk_static``).  For callers that cannot
+    allocate, such as code under graph capture.  q, k, v must already be kernel-ready (head_dim contiguous,
+    16-byte aligned rows); B*H*num_splits*M*(D+2)*4 bytes must fit ``_lib.STATIC_SCRATCH_BYTES``.  Calls that
+    overlap in time on one GPU race on the shared array; calls ordered on one stream do not."""
+    _check_inputs(q, k, v)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    if out.shape != q.shape or out.dtype != q.dtype or out.device != q.device:
+        raise ValueError("out must have the shape, dtype and device of q")
+    for t in (q, k, v):
+        if _kernel_ready(t) is not t:
+            raise ValueError("q, k, v must have head_dim contiguous and 16-byte aligned rows (no copies are made here)")
+    S = int(num_splits) if num_splits else default_num_splits(B, H, N, q.device)
+    a = L.T5ASplitKArgs()
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides3(q), _strides3(k), _strides3(v), _strides3(out)
+    a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
+    a.num_splits, a.sm_scale = S, float(sm_scale)
+    if key_lens is not None:
+        a.key_lens = key_lens.data_ptr()
+        a.key_starts = key_starts.data_ptr() if key_starts is not None else None
+    with _on_device(q):
+        L.check(L.load().t5a_fwd_splitk_static(C.byref(a), _stream(q)))
+    return out
+
+
 def _splitk(q, k, v, bias, sm_scale, num_splits, out_dtype, key_lens=None, key_starts=None):
     _check_inputs(q, k, v)
     B, H, M, D = q.shape
