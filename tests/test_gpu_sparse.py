@@ -215,3 +215,32 @@ def test_splitk_over_padded_memories(gpu_device, dtype, M, N, S):
     assert (right[1] - want[0]).abs().max().item() <= TOL[dtype]
     with pytest.raises(ValueError):
         flash_decoding_attention(dq, dk, dv, None, 1.0, key_starts=ts)
+
+
+@pytest.mark.parametrize("run_len", [1, 2, 3, 5, 16])
+@pytest.mark.parametrize("L,Bl", [(640, 128), (333, 100), (1000, 16), (896, 256), (700, 300)])
+def test_local_with_runs_of_q_tiles(gpu_device, monkeypatch, run_len, L, Bl):
+    """The local pattern's work items are runs of consecutive q tiles (one stream of key tiles through the LDS
+    rings, the distance LUT built once per run); a run may end inside a (batch, head) or cross into the next
+    one.  Every run length must give what the window definition gives, for sequence lengths that are no
+    multiple of anything, with per-sequence lengths, and for windows too wide for the LUT (masked path)."""
+    from turbot5_amd.ops import local_attention_with_fusing_bias
+    monkeypatch.setenv("T5A_RUN_LEN", str(run_len))
+    B, H, D = 2, 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=300 + i, dtype=torch.bfloat16) for i in range(3))
+    table = rnd(32, H, seed=303, scale=1.0)
+    lens = torch.tensor([L, max(1, L - 217)], dtype=torch.int32)
+    dev = [t.to(gpu_device) for t in (q, k, v, table)]
+    out = local_attention_with_fusing_bias(*dev, Bl).float().cpu()
+    out_l = local_attention_with_fusing_bias(*dev, Bl, seq_lens=lens.to(gpu_device)).float().cpu()
+    i = torch.arange(L)[:, None]
+    j = torch.arange(L)[None, :]
+    bias = table[O.relative_position_bucket(j - i, True, 32, 128)].permute(2, 0, 1).unsqueeze(0)
+    bias = bias.masked_fill((j - i).abs() >= Bl, float("-inf"))
+    want = O.basic_attention(q.float(), k.float(), v.float(), bias)
+    assert (out - want).abs().max().item() <= 2e-2
+    for b in range(B):
+        n = int(lens[b])
+        wb = O.basic_attention(q[b:b + 1, :, :n].float(), k[b:b + 1, :, :n].float(), v[b:b + 1, :, :n].float(),
+                               bias[:, :, :n, :n])
+        assert (out_l[b:b + 1, :, :n] - wb).abs().max().item() <= 2e-2, b

@@ -3,6 +3,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <map>
@@ -343,6 +344,47 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     return finish(launch_fwd(p, a->dtype, a->D, kPacked, a->causal != 0, (hipStream_t)stream), "t5a_fwd_varlen");
 }
 
+// Compute units of the current device (cached per device index).
+static int device_compute_units() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static int cus[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    std::lock_guard<std::mutex> g(mu);
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+// Sparse patterns: how many consecutive q tiles of one (batch, head) a workgroup takes.  A q tile of a sparse
+// pattern is only a few steps long, about as long as the set-up of a work item, which a run pays once; longer runs
+// mean fewer workgroups.  Two workgroups fit a compute unit: count the rounds the device needs for the runs and
+// charge every round its q tiles plus one set-up.
+static void choose_runs(FwdParams* p, int mode, int dtype, int D) {
+    p->run_len = 1;
+    p->runs_per_seq = p->tiles_per_seq;
+    const int64_t entries = (int64_t)p->tiles_per_seq * p->H * p->B;   // the (batch, head, q tile) list
+    const bool runs_ok = mode == kLocal && dtype != T5A_F32 && (D == 64 || D == 128);   // the geometries staged by LDS-DMA
+    if (runs_ok) {
+        // as many workgroups as the device holds at once (two per compute unit), each with its share of the list
+        const int64_t slots = 2 * (int64_t)device_compute_units();
+        int64_t rl = (entries + slots - 1) / slots;
+        if (rl > 16) rl = 16;
+        if (rl < 1) rl = 1;
+        p->run_len = (int)rl;
+        // T5A_RUN_LEN=<n>: fixed run length, for tests and measurements
+        if (const char* e = getenv("T5A_RUN_LEN")) {
+            const int forced = atoi(e);
+            if (forced >= 1) p->run_len = forced;
+        }
+    }
+    p->total_items = (int)((entries + p->run_len - 1) / p->run_len);
+}
+
 // Key splits for the global rows of the block pattern: enough (batch, head, split) items to fill the
 // device about twice, at least four key tiles of 64 per split.
 static void global_row_splits(int B, int H, int L, int* nsplit, int* split_rows) {
@@ -425,12 +467,13 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         // pass 1: rows >= G attend [global tokens | own block]
         const int nblk = (a->L + a->block_len - 1) / a->block_len;
         p.tiles_per_seq = nblk * ((a->block_len + 127) / 128);
-        p.total_items = p.tiles_per_seq * a->H * a->B;
+        choose_runs(&p, kBlock, a->dtype, a->D);
         rc = finish(launch_fwd(p, a->dtype, a->D, kBlock, false, s), "t5a_fwd_sparse(block)");
         if (rc || a->aux == 0) return rc;
         // pass 2: the G global queries attend every key; positions are absolute, so M is
         // clipped to G rows of the same tensors (rel = j - i, no end alignment)
         FwdParams g = p;
+        g.run_len = 1;
         g.M = a->aux < a->L ? a->aux : a->L;
         g.N = a->L;
         g.tiles_per_seq = (g.M + 127) / 128;
@@ -462,8 +505,9 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         return finish(launch_fwd(g, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, global rows)");
     }
     p.tiles_per_seq = (a->L + 127) / 128;
-    p.total_items = p.tiles_per_seq * a->H * a->B;
-    return finish(launch_fwd(p, a->dtype, a->D, a->pattern == T5A_PATTERN_LOCAL ? kLocal : kTGlobal, false, s), "t5a_fwd_sparse");
+    const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? kTGlobal : (a->block_len <= kMaxLutWindow ? kLocal : kLocalWide);
+    choose_runs(&p, mode, a->dtype, a->D);
+    return finish(launch_fwd(p, a->dtype, a->D, mode, false, s), "t5a_fwd_sparse");
 }
 
 int64_t t5a_splitk_workspace_bytes(int32_t B, int32_t H, int32_t M, int32_t D, int32_t num_splits) {

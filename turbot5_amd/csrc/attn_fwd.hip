@@ -115,7 +115,11 @@ constexpr int NTHREADS = 256;
 // every tile.  Probabilities then reach 2^limit: bf16 and fp32 have the exponent range for 2^24 (sums
 // and outputs are fp32 and are divided by the row sum at the end); fp16 tops out at 65504, hence 2^14.
 template <typename T> constexpr float raise_limit() { return sizeof(T) == 2 && !__is_same(T, __bf16) ? 14.0f : 24.0f; }
-constexpr int kWorkgroupsPerCU = 2;   // 72 KB of LDS and 256 registers per lane each
+// a row whose first scores (base-2 units) are at least this keeps its running max at 0 (fp16 probabilities lose
+// their precision below 2^-14, so fp16 rows start at their maximum unless it is close to 0)
+template <typename T> constexpr float start_floor() { return sizeof(T) == 2 && !__is_same(T, __bf16) ? -8.0f : -100.0f; }
+constexpr int kWorkgroupsPerCU = 2;
+   // 72 KB of LDS and 256 registers per lane each
 
 // table element from its bits (zero-extended for the 16-bit types)
 __device__ __forceinline__ float table_value(unsigned raw, int dtype) {
@@ -239,7 +243,7 @@ struct Geometry {
     static __device__ __forceinline__ int vrow_swz(int key) { return D == 128 ? (key & 3) << 2 : ((key >> 1) & 1) << 2; }
 };
 
-template <typename T, int D, int MODE, bool CAUSAL>
+template <typename T, int D, int MODE, bool CAUSAL, bool EXACT>
 __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkgroupsPerCU) void fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using G = Geometry<T, D>;
@@ -252,14 +256,20 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     constexpr int ES = sizeof(T);
     constexpr int BN = G::BN, NT = G::NT;
     constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
+    constexpr bool LOCAL = MODE == kLocal || MODE == kLocalWide;   // sliding window, one segment
+    // Sparse patterns, LDS-DMA geometries: a work item is a RUN of consecutive q tiles of one (batch, head).  Their
+    // key tiles form one stream through the LDS rings (the requests for the next q tile's first tiles go out during
+    // the last steps of the current one) and the distance LUT is built once per run; a q tile of a sparse pattern
+    // is only a few steps long, so that its set-up would otherwise cost as much as its steps.
+    constexpr bool RUNS = MODE == kLocal && G::DMA;
     // head_dim 64, 16-bit types: the Q rows are staged through LDS by LDS-DMA as well (see the prologue)
     constexpr bool QDMA = G::DMA && D == 64;
     // 16-bit inputs, two ways to apply sm_scale * log2(e).  Default: Q is pre-multiplied and rounded back to the
     // input type, which puts a relative error of 2^-9 (bf16; 2^-12 for fp16) on every term of a score and costs
     // nothing per tile.  exact_scale: the Q fragments stay as loaded, the accumulator input is divided by the
     // factor and the fp32 product is multiplied by it: one more vector multiply per score (about 11 % of the
-    // run time at head_dim 64).  Wavefront-uniform, decided once per launch.
-    const bool exact = !F32 && p.exact_scale != 0;
+    // run time at head_dim 64).  A template parameter: as a run-time switch it cost the default path 2-3 %.
+    constexpr bool exact = EXACT && !F32;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr bool DMA = G::DMA;
@@ -309,6 +319,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (w >= p.total_items) return;
     }
 
+    // RUNS: the work item is run_len consecutive entries of the (batch, head, q tile) list.  The part of it that
+    // lies in one (batch, head) is one pass of the loop below (set-up, then its q tiles as one stream); a run that
+    // crosses into the next (batch, head) starts over there with a new set-up.
+    int run_left = 1, run_next = 0;
+    if constexpr (RUNS) {
+        run_next = w * p.run_len;
+        run_left = min(p.run_len, p.tiles_per_seq * p.H * p.B - run_next);
+    }
+    for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     int n_side = p.n_side;   // side tokens of this item's sequence (transient-global)
     int64_t q_off, k_off, v_off, o_off, lse_off;
@@ -346,8 +365,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         lse_off = (int64_t)qs * p.lse_sr + (int64_t)h * p.lse_sh;
     } else {
         // unsigned arithmetic: the divisions are scalar code on every workgroup's critical path
-        unsigned bh = (unsigned)w / (unsigned)p.tiles_per_seq;
-        qt = (int)((unsigned)w - bh * (unsigned)p.tiles_per_seq);
+        const unsigned entry = RUNS ? (unsigned)run_next : (unsigned)w;
+        unsigned bh = entry / (unsigned)p.tiles_per_seq;
+        qt = (int)(entry - bh * (unsigned)p.tiles_per_seq);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
         if (MODE == kDense && p.nsplit > 1) {
             const unsigned g = bh / (unsigned)p.nsplit;
@@ -361,7 +381,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         // windowed patterns on a right-padded batch: the keys of a sequence end at its length; positions are
         // the row indices, so nothing else changes (rows past the length see what is left of their window).
         // Its side tokens are the full blocks of that length, the rest of its tokens joining the last one.
-        if ((MODE == kLocal || MODE == kTGlobal) && p.len_k != nullptr) {
+        if ((LOCAL || MODE == kTGlobal) && p.len_k != nullptr) {
             Nseq = max(0, min(p.N, p.len_k[b]));
             if (MODE == kTGlobal) n_side = min(p.n_side, Nseq / p.aux);
         }
@@ -380,18 +400,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     const T* qp = reinterpret_cast<const T*>(p.q) + q_off;
     T* op = reinterpret_cast<T*>(p.o) + o_off;
 
-    // query rows of this tile: [i0, row_end); rows below row_lo are computed but not stored
-    int i0, row_end, row_lo = 0, blk = 0;
-    if (MODE == kBlock) {
-        const int tpb = (p.block_len + BM - 1) / BM;
-        blk = qt / tpb;
-        i0 = blk * p.block_len + (qt - blk * tpb) * BM;
-        row_end = min(Mseq, (blk + 1) * p.block_len);
-        row_lo = p.aux;   // the first G rows belong to the global-query pass
-    } else {
-        i0 = qt * BM;
-        row_end = Mseq;
-    }
+    // q tiles of this item: one, or a run of consecutive ones (RUNS)
+    int qt_count = 1;
+    if constexpr (RUNS) qt_count = min(run_left, p.tiles_per_seq - qt);
+    const int qt_last = qt + qt_count;   // one past the last q tile of this pass
+    // query rows of the current q tile: [i0, row_end); rows below row_lo are computed but not stored
+    int i0 = 0, row_end = 0, row_lo = 0, blk = 0;
+    const int tpb = MODE == kBlock ? (p.block_len + BM - 1) / BM : 1;   // q tiles per block (block pattern)
+    if (MODE == kBlock) row_lo = p.aux;   // the first G rows belong to the global-query pass
     const int P = p.align_end ? Nseq - Mseq : -key0;   // query position minus row index, in this item's key numbering
 
     // ---------------------------------------------------------------- key segments
@@ -412,11 +428,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     seg_start[0] = 0; seg_end[0] = 0;
     seg_start[1] = seg_end[1] = seg_lend[1] = 0; seg_kind[1] = 0; seg_win[1] = 0;
     seg_kind[0] = 0; seg_win[0] = 0; seg_lend[0] = Nseq;
-    if (DENSE) {
-        seg_end[0] = CAUSAL ? max(0, min(Nseq, i0 + BM + P)) : Nseq;
-    } else if (MODE == kLocal || MODE == kTGlobal) {
-        seg_start[0] = max(0, i0 - p.block_len + 1);
-        seg_end[0] = min(Nseq, min(i0 + BM, Mseq) - 1 + p.block_len);
+    if (LOCAL || MODE == kTGlobal) {
         seg_win[0] = 1;
         if (MODE == kTGlobal) {
             nseg = 2;
@@ -425,23 +437,68 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             seg_ksr[1] = (int)p.sk_sr * ES; seg_vsr[1] = (int)p.sv_sr * ES;
             seg_end[1] = n_side; seg_lend[1] = n_side; seg_kind[1] = 2;
         }
-    } else {  // kBlock
+    } else if (MODE == kBlock) {
         nseg = 2;
         seg_end[0] = p.aux; seg_kind[0] = 1;
-        seg_start[1] = blk * p.block_len;
-        seg_end[1] = blk == 0 ? p.block_len - p.aux : (blk + 1) * p.block_len;
         seg_lend[1] = Nseq;
     }
-    int seg_nt[2];
-    seg_nt[0] = max(0, seg_end[0] - seg_start[0] + BN - 1) / BN;
-    seg_nt[1] = nseg > 1 ? max(0, seg_end[1] - seg_start[1] + BN - 1) / BN : 0;
-    const int ntiles = seg_nt[0] + seg_nt[1];
+    // The part of the geometry that changes from one q tile to the next.  RUNS: every q tile of the run has the
+    // same number of tiles per segment (seg_nt): the window starts where it starts even when that is before key 0,
+    // and a block's segment spans a whole block; tiles outside the keys that exist read as zeros and are skipped
+    // or masked.
+    int seg_nt[2] = {0, 0};
+    auto set_qtile = [&](int q_tile) {
+        if (MODE == kBlock) {
+            blk = q_tile / tpb;
+            i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
+            row_end = min(Mseq, (blk + 1) * p.block_len);
+            seg_start[1] = blk * p.block_len;
+            seg_end[1] = blk == 0 ? p.block_len - p.aux : (blk + 1) * p.block_len;
+        } else {
+            i0 = q_tile * BM;
+            row_end = Mseq;
+        }
+        if (DENSE) {
+            seg_end[0] = CAUSAL ? max(0, min(Nseq, i0 + BM + P)) : Nseq;
+        } else if (LOCAL || MODE == kTGlobal) {
+            seg_start[0] = RUNS ? i0 - p.block_len + 1 : max(0, i0 - p.block_len + 1);
+            seg_end[0] = min(Nseq, min(i0 + BM, Mseq) - 1 + p.block_len);
+        }
+    };
+    // first row and end of the rows of any q tile of this (batch, head)
+    auto qtile_rows = [&](int q_tile, int& first, int& end) {
+        if (MODE == kBlock) {
+            const int bk = q_tile / tpb;
+            first = bk * p.block_len + (q_tile - bk * tpb) * BM;
+            end = min(Mseq, (bk + 1) * p.block_len);
+        } else {
+            first = q_tile * BM;
+            end = Mseq;
+        }
+    };
+    set_qtile(qt);
+    if constexpr (RUNS) {
+        if (MODE == kBlock) { seg_nt[0] = (p.aux + BN - 1) / BN; seg_nt[1] = (p.block_len + BN - 1) / BN; }
+        else { seg_nt[0] = (BM + 2 * p.block_len - 2 + BN - 1) / BN; seg_nt[1] = nseg > 1 ? (n_side + BN - 1) / BN : 0; }
+    } else {
+        seg_nt[0] = max(0, seg_end[0] - seg_start[0] + BN - 1) / BN;
+        seg_nt[1] = nseg > 1 ? max(0, seg_end[1] - seg_start[1] + BN - 1) / BN : 0;
+    }
+    // an even number of tiles per q tile keeps the two score buffers of the pipeline in step from one q tile of a
+    // run to the next (the extra tile lies past its segment's end and is skipped)
+    if (RUNS && ((seg_nt[0] + seg_nt[1]) & 1)) {   // (no run-time index: that would move the array to scratch memory)
+        if (nseg > 1) seg_nt[1] += 1; else seg_nt[0] += 1;
+    }
+    const int ntiles = seg_nt[0] + seg_nt[1];   // tiles of one q tile
+    int tbase = 0;                               // tiles of the run's earlier q tiles (the ring stages count on)
     __amdgpu_buffer_rsrc_t seg_krs[2], seg_vrs[2];
     u32x4 seg_krw[2], seg_vrw[2];
     int seg_kbytes0 = 0, seg_vbytes0 = 0;   // readable bytes of segment 0
 #pragma unroll
     for (int sg = 0; sg < 2; ++sg) {
-        const int rows = min(seg_lend[sg], seg_end[sg]);   // rows at or past this read as zero
+        // rows at or past this read as zero.  RUNS: one descriptor per tensor for the whole run -- all the keys of
+        // the (batch, head); what a q tile must not see of them is masked
+        const int rows = RUNS ? (sg == 0 || MODE == kBlock ? Nseq : n_side) : min(seg_lend[sg], seg_end[sg]);
         const unsigned kb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_ksr[sg] + D * ES : 0u;
         const unsigned vb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_vsr[sg] + D * ES : 0u;
         seg_krs[sg] = make_rsrc(seg_k[sg], kb);
@@ -452,9 +509,23 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
+    // tile t of the current q tile -> segment and first key.  RUNS: t may run past the q tile's last tile into the
+    // following q tiles of the run (requests are issued up to four tiles ahead); returns false past the run's end.
     auto tile_of = [&](int t, int& sg, int& j0) {
-        sg = t >= seg_nt[0] ? 1 : 0;
-        j0 = (sg ? seg_start[1] : seg_start[0]) + (t - (sg ? seg_nt[0] : 0)) * BN;
+        if constexpr (RUNS) {
+            int ahead = 0;
+            while (t >= ntiles) { t -= ntiles; ++ahead; }
+            const int q_tile = qt + ahead;
+            sg = t >= seg_nt[0] ? 1 : 0;
+            const int ts = t - (sg ? seg_nt[0] : 0);
+            if (MODE == kBlock) j0 = sg ? (q_tile / tpb) * p.block_len + ts * BN : ts * BN;
+            else j0 = sg ? ts * BN : q_tile * BM - p.block_len + 1 + ts * BN;
+            return q_tile < qt_last;
+        } else {
+            sg = t >= seg_nt[0] ? 1 : 0;
+            j0 = (sg ? seg_start[1] : seg_start[0]) + (t - (sg ? seg_nt[0] : 0)) * BN;
+            return true;
+        }
     };
     // LDS-DMA staging: a wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses
     // (8 rows of 128 bytes); the XOR swizzles are applied on the SOURCE side: the lane that owns
@@ -462,10 +533,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // segment are out of the buffer's range and arrive as zeros.
     auto dma_tile = [&](int t, bool is_v, int stage = -1) {
         if constexpr (DMA) {
-            int sg, j0; tile_of(t, sg, j0);
-            const u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
+            int sg, j0;
+            const bool in_run = tile_of(t, sg, j0);
+            u32x4 rs = is_v ? (sg ? seg_vrw[1] : seg_vrw[0]) : (sg ? seg_krw[1] : seg_krw[0]);
+            if (!in_run) rs[2] = 0u;   // nothing is readable: the request fills its stage with zeros
             const int sr = is_v ? (sg ? seg_vsr[1] : seg_vsr[0]) : (sg ? seg_ksr[1] : seg_ksr[0]);
-            if (stage < 0) stage = is_v ? t % NSV : t % NSK;
+            if (stage < 0) stage = is_v ? (tbase + t) % NSV : (tbase + t) % NSK;
             const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
 #pragma unroll
             for (int c = 0; c < G::SPW; ++c) {
@@ -523,11 +596,28 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
     };
     // ---------------------------------------------------------------- Q fragments: loads first
-    const int iw0 = i0 + wave * 32;      // first row of this wavefront
-    const int iw1 = iw0 + 31;
-    const int irow = iw0 + lr;           // this lane's query row
-    const bool row_ok = irow < row_end;
+    int iw0 = i0 + wave * 32;      // first row of this wavefront
+    int iw1 = iw0 + 31;
+    int irow = iw0 + lr;           // this lane's query row
+    bool row_ok = irow < row_end;
     v8 qf[KS];
+    // RUNS: the Q rows of the run's NEXT q tile, requested a whole q tile ahead (plain loads: they have landed long
+    // before the switch, where the only cost left is the compiler's wait for everything in flight)
+    v8 qn[RUNS ? KS : 1];
+    auto prefetch_q = [&](int q_tile) {
+        if constexpr (RUNS) {
+            int first, end;
+            qtile_rows(q_tile, first, end);
+            const int row = first + wave * 32 + lr;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qn[s][e] = (T)0.0f;
+                if (q_tile < qt_last && row < end)
+                    qn[s] = *reinterpret_cast<const v8*>(qp + (int64_t)row * p.q_sr + 16 * s + 8 * hh);
+            }
+        }
+    };
     f32x4 qraw[F32 ? D / 4 : 1];
     if constexpr (F32) {
 #pragma unroll
@@ -546,8 +636,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
 
     // ---------------------------------------------------------------- bias LUT
     const bool has_bias = p.table != nullptr;
-    const bool has_lut = has_bias || CAUSAL;
-    const int sat = has_bias ? p.bs.sat : 0;
+    // Sliding window folded into the LUT (local pattern, windows up to kMaxLutWindow): the window is a function
+    // of the distance alone, so the LUT holds -inf from the window's edge on and reaches LUT_PAD past it.
+    // No tile then needs a per-element window mask, and every tile that is not skipped is a LUT tile.
+    constexpr bool win_lut = MODE == kLocal;   // the host picks kLocal for windows up to kMaxLutWindow
+    const bool has_lut = has_bias || CAUSAL || win_lut;
+    const int sat_bias = has_bias ? p.bs.sat : 0;
+    const int sat = win_lut ? max(sat_bias, p.block_len) : sat_bias;   // distance from which the LUT is constant
     const int padl = sat + LUT_PAD;                       // LUT index of rel = 0
     const int quads = lut_quads(sat, CAUSAL);
     const int qlen = 4 * quads;
@@ -564,7 +659,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // register written by a load issued from inline assembly is still in flight and may copy it too early.
     const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
     const bool col_in_lanes = nbt <= 64;
-    const bool lut_cached = has_bias && p.lut_global != nullptr;   // the host checked qlen <= 512
+    // (a per-table buffer holds the plain LUTs: not the ones with a window folded in)
+    const bool lut_cached = has_bias && p.lut_global != nullptr && !win_lut;   // the host checked qlen <= 512
     const int col_esize = p.table_dtype == T5A_F32 ? 4 : 2;
     // byte offset of this lane's bucket in the table, from the 4-byte aligned address at or below its start
     const unsigned col_misalign = (unsigned)(reinterpret_cast<uintptr_t>(p.table) & 3);
@@ -643,7 +739,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
     } else if (has_lut) {
         lut_fill<CAUSAL>(lut, p.bs, p.table, p.table_dtype, p.t_sbucket, p.t_shead, h, has_bias, tcol, col_in_lanes,
-                         padl, qlen, tid, NTHREADS);
+                         padl, qlen, tid, NTHREADS, win_lut ? p.block_len : 0x7fffffff);
     }
     if (D < 32) {  // the part of V past head_dim feeds the MFMA: keep it zero
         for (int idx = tid; idx < NSV * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
@@ -800,19 +896,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         d_ts = iw0 >= row_end ? 0 : (CAUSAL ? (qhi < 0 ? 0 : qhi / BN + 1) : 0x7fffffff);  // skipped from here
         d_tm = seg_end[0] / BN;                                // tiles from here on straddle the segment end
     }
-    auto classify = [&](int t) {
+    // sparse patterns: the class of a tile from the geometry of the current q tile (a few dozen scalar instructions)
+    auto classify_sparse = [&](int t) {
         TileClass c;
         c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
         if (t >= ntiles) return c;
-        if (DENSE) {
-            c.j0 = t * BN;
-            c.skip = t >= d_ts;
-            const bool left_sat = t < d_tl, right_sat = t >= d_tr;
-            c.use_lut = has_lut && !(left_sat || right_sat);
-            c.need_mask = t >= d_tm;
-            c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
-            return c;
-        }
         tile_of(t, c.sg, c.j0);
         const int kind = (c.sg ? seg_kind[1] : seg_kind[0]);
         const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
@@ -827,9 +915,54 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const bool left_sat = rel_max <= -sat && (!CAUSAL || rel_max <= 0);
         const bool right_sat = !CAUSAL && rel_min >= sat;
         c.use_lut = has_lut && !(left_sat || right_sat);
-        c.need_mask = c.j0 + BN > (c.sg ? seg_end[1] : seg_end[0]);
-        if (win) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
+        if constexpr (win_lut) c.use_lut = true;   // (a tile beyond the window's edge is skipped, never constant)
+        const int s_end = c.sg ? seg_end[1] : seg_end[0];
+        c.need_mask = c.j0 + BN > s_end;
+        if constexpr (RUNS) {   // tiles before key 0 or past the end of the segment exist here (same count for every q tile)
+            c.skip = c.skip || c.j0 >= s_end || c.j0 + BN <= 0;
+            c.need_mask = c.need_mask || c.j0 < 0;
+        }
+        if (win && !win_lut) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
         c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
+        if constexpr (win_lut) c.side = 0;
+        return c;
+    };
+    // ... evaluated once per q tile into bit sets (bit t = tile t): the steps only test bits.  Q tiles of more than
+    // 64 tiles (transient-global over very long inputs) classify every tile when they reach it.
+    unsigned long long cls_skip = 0, cls_mask = 0, cls_lut = 0, cls_right = 0;
+    const bool cls_bits = RUNS && ntiles <= 64;   // (with many tiles per q tile, classifying them up front costs more than it saves)
+    auto fill_classes = [&]() {
+        cls_skip = cls_mask = cls_lut = cls_right = 0;
+        if (!cls_bits) return;
+        for (int t = 0; t < ntiles; ++t) {
+            const TileClass c = classify_sparse(t);
+            const unsigned long long bit = 1ull << t;
+            if (c.skip) cls_skip |= bit;
+            if (c.need_mask) cls_mask |= bit;
+            if (c.use_lut) cls_lut |= bit;
+            if (c.side == 2) cls_right |= bit;
+        }
+    };
+    auto classify = [&](int t) {
+        TileClass c;
+        c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
+        if (t >= ntiles) return c;
+        if (DENSE) {
+            c.j0 = t * BN;
+            c.skip = t >= d_ts;
+            const bool left_sat = t < d_tl, right_sat = t >= d_tr;
+            c.use_lut = has_lut && !(left_sat || right_sat);
+            c.need_mask = t >= d_tm;
+            c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
+            return c;
+        }
+        if (!cls_bits) return classify_sparse(t);
+        tile_of(t, c.sg, c.j0);
+        const unsigned long long bit = 1ull << t;
+        c.skip = (cls_skip & bit) != 0;
+        c.need_mask = (cls_mask & bit) != 0;
+        c.use_lut = win_lut || (cls_lut & bit) != 0;
+        c.side = (!win_lut && has_bias && !c.use_lut && !c.skip) ? ((cls_right & bit) != 0 ? 2 : 1) : 0;
         return c;
     };
 
@@ -843,6 +976,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     float l_run = 0.f;       // running sum over this lane's half of the keys (two partial sums)
     float l_alt = 0.f;
     bool started = false;    // a finite score has been seen for this row
+    // wavefront-uniform: every row's running max is still exactly 0 (rows start there unless their first scores
+    // are huge or tiny), so a LUT tile's accumulator input is the LUT entry itself, without a subtraction
+    bool m_zero = true;
     // accumulator input of tiles with a constant bias: (constant - m_run) in all 16 slots.  It is
     // rewritten in ONE place per step, when the running max was raised or the tiles crossed to
     // the other saturated side, so the common path carries no copies of it.
@@ -883,16 +1019,27 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const int e0 = c.j0 + 4 * hh - qpos + padl;
             const float* lb = lut + (e0 & 3) * qlen;
             const int y0 = e0 >> 2;
+            if (!DENSE && m_zero && !exact) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+                for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int y = y0 + 8 * nt + 2 * g;   // always inside the LUT, see LUT_PAD
-                    const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * (y0 + 8 * nt + 2 * g));
 #pragma unroll
-                    for (int x = 0; x < 4; ++x)
-                        st[nt][4 * g + x] = __builtin_fmaf(bq[x], inv_c1, m_neg);
-                }
+                        for (int x = 0; x < 4; ++x) st[nt][4 * g + x] = bq[x];
+                    }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int y = y0 + 8 * nt + 2 * g;   // always inside the LUT, see LUT_PAD
+                        const f32x4 bq = *reinterpret_cast<const f32x4*>(lb + 4 * y);
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            st[nt][4 * g + x] = __builtin_fmaf(bq[x], inv_c1, m_neg);
+                    }
+            }
         }
         if constexpr (F32) {
             const T* ks = Ks + buf * K_TILE;
@@ -920,8 +1067,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     for (int s = 1; s < KS; ++s) st[nt] = E::mfma(ka[nt][s], qf[s], st[nt]);
                 }
             }
-            if (exact) {
-                asm volatile("");   // a real branch around the multiplies, not 32 selects
+            if constexpr (exact) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -934,7 +1080,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto softmax_head = [&](const TileClass& c, f32x16 (&st)[NT]) {
         if (c.need_mask) {   // keys past the end of the segment, or outside the window
             const int s_end = (c.sg ? seg_end[1] : seg_end[0]);
-            const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
+            const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0 && !win_lut;
             const int qpos = lane_qpos(c.sg);
             // this lane's row sees the keys [lo, hi): one subtraction and one unsigned compare per element
             const int lo = win ? max(0, qpos - p.block_len + 1) : 0;
@@ -965,11 +1111,17 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (__any((mh > raise_limit<T>()) || (!started && mh > -INFINITY))) {
             asm volatile("");   // keep this rare block a real branch
             const float mx = xhalf_max(mh);
-            const bool raise = (mx > raise_limit<T>()) || (!started && mx > -INFINITY);
+            // a row's first finite scores: the running max stays at 0 when they are moderate (probabilities
+            // between 2^-100 and 2^24 are safe in bf16 / fp32 and fp16's limit is lower still), else it goes to them
+            // (sparse patterns only, where most tiles take their bias from the LUT; dense rows go to their first
+            // maximum: there the zero start costs long sequences 1 %)
+            const bool fresh = !started && mx > -INFINITY;
+            const bool raise = (mx > raise_limit<T>()) || (fresh && (DENSE || mx < start_floor<T>()));
             const float delta = raise ? mx : 0.f;
             const float scale = started ? __builtin_amdgcn_exp2f(-delta) : 0.f;
             m_run += delta;
-            started = started || raise;
+            started = started || fresh;
+            m_zero = m_zero && !__any(raise);
             l_run *= scale;
             l_alt *= scale;
 #pragma unroll
@@ -1075,7 +1227,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // "at most two steps' worth outstanding" before the barrier means the tiles of the next step
     // have landed.
     f32x16 sta[NT], stb[NT];
+    fill_classes();
     TileClass tc = classify(0);
+    const bool first_interior = LOCAL && seg_start[0] >= 0 && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
     if constexpr (QDMA) {
         // K0 and V0 landed before the barrier that published the LUT
     } else {
@@ -1099,8 +1253,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (QDMA) dma_tile(3, false);         // K3, into the stage that held the Q rows of two wavefronts
 
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
-        const int kbuf_next = DMA ? (t + 1) % NSK : (t + 1) & 1;
-        const int vbuf = DMA ? t % NSV : t & 1;
+        const int kbuf_next = DMA ? (tbase + t + 1) % NSK : (t + 1) & 1;
+        const int vbuf = DMA ? (tbase + t) % NSV : t & 1;
         if constexpr (DMA) {
             dma_tile(t + 4, false);
             dma_tile(t + 3, true);
@@ -1150,6 +1304,10 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // number of consecutive tiles from t on that are neither skipped nor masked
     auto plain_run = [&](int t) {
         if (DENSE) return max(0, min(min(d_ts, d_tm), ntiles) - t);
+        if (cls_bits) {
+            const unsigned long long bad = (cls_skip | cls_mask) >> t;
+            return min(bad != 0 ? (int)__builtin_ctzll(bad) : 64, ntiles - t);
+        }
         int n = 0;
         for (; t + n < ntiles; ++n) {
             const TileClass c = classify(t + n);
@@ -1158,40 +1316,34 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         return n;
     };
 
-    int t = 0;
-    while (t < ntiles) {
-        if (DMA && (t & 3) == 0) {
-            // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5.  When the run reaches the
-            // last tile, the final fast step forms an S product for a tile that does not exist (its K
-            // stage was filled with zeros) and nobody consumes it, so the run may end exactly there.
-            const int run = plain_run(t);
-            int quads = (t + run >= ntiles ? run : run - 1) >> 2;
-            if (quads > 0) {
-                tc = classify(t);
-                if constexpr (DENSE) cursor_seek(t + 4, t + 3);
+    // rows of the current q tile: normalise, convert, store (and the log-sum-exp when asked for)
+    auto store_rows = [&]() {
+        const float l_tot = xhalf_sum(l_run + l_alt);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (MODE == kDense && p.nsplit > 1) {
+            // partial result of a key split: normalised row in fp32, weight 1 (0: no visible key) and log-sum-exp
+            if (row_ok) {
+                const int64_t prow = (((int64_t)b * p.H + h) * p.nsplit + split) * p.M + irow;
+                float* orow = p.part_o + prow * D;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int d0 = 32 * dt + 8 * g + 4 * hh;
+                        if (d0 < D) {
+                            f32x4 x;
+#pragma unroll
+                            for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
+                            *reinterpret_cast<f32x4*>(orow + d0) = x;
+                        }
+                    }
+                if (hh == 0) {
+                    p.part_l[prow] = l_tot > 0.f ? 1.f : 0.f;
+                    p.part_m[prow] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
+                }
             }
-            while (quads > 0) {
-                fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
-                fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
-                fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
-                fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
-                --quads; t += 4;
-            }
-            if (t >= ntiles) break;
-        }
-        step(t, sta, stb);
-        if (t + 1 < ntiles) step(t + 1, stb, sta);
-        t += 2;
-    }
-
-    // ---------------------------------------------------------------- epilogue
-    const float l_tot = xhalf_sum(l_run + l_alt);
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (MODE == kDense && p.nsplit > 1) {
-        // partial result of a key split: normalised row in fp32, weight 1 (0: no visible key) and log-sum-exp
-        if (row_ok) {
-            const int64_t prow = (((int64_t)b * p.H + h) * p.nsplit + split) * p.M + irow;
-            float* orow = p.part_o + prow * D;
+        } else if (row_ok && irow >= row_lo) {
+            T* orow = op + (int64_t)irow * p.o_sr;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -1201,45 +1353,115 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                         f32x4 x;
 #pragma unroll
                         for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
-                        *reinterpret_cast<f32x4*>(orow + d0) = x;
+                        if constexpr (F32) *reinterpret_cast<f32x4*>(orow + d0) = x;
+                        else *reinterpret_cast<v4*>(orow + d0) = __builtin_convertvector(x, v4);
                     }
                 }
-            if (hh == 0) {
-                p.part_l[prow] = l_tot > 0.f ? 1.f : 0.f;
-                p.part_m[prow] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
+            if (p.lse != nullptr && hh == 0) {
+                const float ln2 = 0.6931471805599453f;
+                p.lse[lse_off + (int64_t)irow * p.lse_sr] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * ln2 : -INFINITY;
             }
         }
-    } else if (row_ok && irow >= row_lo) {
-        T* orow = op + (int64_t)irow * p.o_sr;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d0 = 32 * dt + 8 * g + 4 * hh;
-                if (d0 < D) {
-                    f32x4 x;
-#pragma unroll
-                    for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
-                    if constexpr (F32) *reinterpret_cast<f32x4*>(orow + d0) = x;
-                    else *reinterpret_cast<v4*>(orow + d0) = __builtin_convertvector(x, v4);
+    };
+
+    if constexpr (RUNS) prefetch_q(qt + 1);
+    bool interior = first_interior;   // the current q tile's classes hold for any q tile away from the ends of the sequence
+    for (;;) {
+        int t = 0;
+        while (t < ntiles) {
+            if (DMA && ((tbase + t) & 3) == 0) {
+                // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5.  When the run reaches the
+                // last tile, the final fast step forms an S product for a tile that does not exist (its K
+                // stage holds zeros or a tile of the next q tile) and nobody consumes it, so the run may end
+                // exactly there.
+                const int run = plain_run(t);
+                int quads = (t + run >= ntiles ? run : run - 1) >> 2;
+                if (quads > 0) {
+                    tc = classify(t);
+                    if constexpr (DENSE) cursor_seek(t + 4, t + 3);
                 }
+                while (quads > 0) {
+                    fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
+                    fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
+                    fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
+                    fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
+                    --quads; t += 4;
+                }
+                if (t >= ntiles) break;
             }
-        if (p.lse != nullptr && hh == 0) {
-            const float ln2 = 0.6931471805599453f;
-            p.lse[lse_off + (int64_t)irow * p.lse_sr] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * ln2 : -INFINITY;
+            step(t, sta, stb);
+            if (t + 1 < ntiles) step(t + 1, stb, sta);
+            t += 2;
         }
+        if constexpr (!RUNS) {
+            store_rows();
+            break;
+        } else {
+            // ------------------------------------------------------------ next q tile of the run
+            // Its first tiles are in the rings already or on their way (the steps above requested them), the LUT
+            // stays, its Q rows were requested a q tile ago.  What is left of a work item's set-up: the geometry
+            // and the first score product.
+            if (qt + 1 >= qt_last) { store_rows(); break; }
+#pragma unroll
+            for (int s = 0; s < KS; ++s) qf[s] = qn[s];
+            store_rows();
+            ++qt;
+            tbase += ntiles;
+            set_qtile(qt);
+            iw0 = i0 + wave * 32; iw1 = iw0 + 31; irow = iw0 + lr; row_ok = irow < row_end;
+            prefetch_q(qt + 1);
+            if (!exact) {
+#pragma unroll
+                for (int s = 0; s < KS; ++s)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)qf[s][e] * p.c1);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
+            m_run = 0.f; l_run = 0.f; l_alt = 0.f; started = false; m_zero = true;
+            side_cur = 0; cb_cur = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) cm[r] = 0.f;
+            // away from the ends of the sequence every q tile of the local pattern has the same classes
+            const bool was_interior = interior;
+            interior = LOCAL && seg_start[0] >= 0 && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+            if (!(interior && was_interior)) fill_classes();
+            tc = classify(0);
+            if (tc.side != 0) refill_cm(tc.side);
+            if (!tc.skip) {
+                v8 ka0[NT][KS];
+                read_k(tbase % NSK, ka0);
+                compute_s(tc, tbase % NSK, ka0, sta);
+            }
+            barrier_lds_only();   // the first step's request overwrites the K stage this product was read from
+        }
+    }
+    if constexpr (!RUNS) {
+        break;
+    } else {
+        run_left -= qt_count;
+        run_next += qt_count;
+        if (run_left <= 0) break;
+        // the run goes on in the next (batch, head): nothing of this one may still be on its way into the rings
+        // (the last steps requested tiles past the end: zeros), and every wavefront must be done with the LUT
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        __syncthreads();
+    }
     }
 }
 
 // ------------------------------------------------------------------------ launch
-template <typename T, int D, int MODE, bool CAUSAL>
-static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
-    const int sat = p.table != nullptr ? p.bs.sat : 0;
+template <typename T, int D, int MODE, bool CAUSAL, bool EXACT>
+static hipError_t launch_exact(const FwdParams& p, hipStream_t stream) {
+    int sat = p.table != nullptr ? p.bs.sat : 0;
+    if (MODE == kLocal) sat = std::max(sat, p.block_len);   // window folded into the LUT
     // the LUT image rounded up to 1 KB (its LDS-DMA requests are that long) and 256 bytes per wavefront
     // for the table column
     const size_t lut_bytes = (((size_t)16 * lut_quads(sat, CAUSAL) * sizeof(float) + 1023) & ~(size_t)1023) + 1024;
     const size_t smem = Geometry<T, D>::kTileBytes + lut_bytes;
-    auto kern = fwd_kernel<T, D, MODE, CAUSAL>;
+    auto kern = fwd_kernel<T, D, MODE, CAUSAL, EXACT>;
     // per instantiation and device: largest dynamic LDS size already allowed (the attribute belongs to the
     // function as loaded on one device)
     constexpr int kMaxDevices = 64;
@@ -1269,12 +1491,21 @@ static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+template <typename T, int D, int MODE, bool CAUSAL>
+static hipError_t launch_one(const FwdParams& p, hipStream_t stream) {
+    if constexpr (sizeof(T) == 2) {
+        if (p.exact_scale != 0) return launch_exact<T, D, MODE, CAUSAL, true>(p, stream);
+    }
+    return launch_exact<T, D, MODE, CAUSAL, false>(p, stream);
+}
+
 template <typename T, int D>
 static hipError_t launch_mode(const FwdParams& p, int mode, bool causal, hipStream_t s) {
     switch (mode) {
         case kDense: return causal ? launch_one<T, D, kDense, true>(p, s) : launch_one<T, D, kDense, false>(p, s);
         case kPacked: return causal ? launch_one<T, D, kPacked, true>(p, s) : launch_one<T, D, kPacked, false>(p, s);
         case kLocal: return launch_one<T, D, kLocal, false>(p, s);
+        case kLocalWide: return launch_one<T, D, kLocalWide, false>(p, s);
         case kBlock: return launch_one<T, D, kBlock, false>(p, s);
         case kTGlobal: return launch_one<T, D, kTGlobal, false>(p, s);
     }

@@ -43,12 +43,13 @@ __device__ __forceinline__ float load_table(const void* table, int dtype, int64_
 }
 
 // Fills the four shifted copies of one head's LUT: copy a, slot i holds the bias of distance i + a - padl,
-// already multiplied by log2(e); future keys hold -inf when CAUSAL.  `tcol`: when col_in_lanes, lane b of
+// already multiplied by log2(e); future keys hold -inf when CAUSAL, distances of `window` and more hold -inf.  `tcol`: when col_in_lanes, lane b of
 // every wavefront holds the table value of bucket b (times log2 e).  Every thread of the workgroup must call.
 template <bool CAUSAL>
 __device__ __forceinline__ void lut_fill(float* lut, const BucketSpec& bs, const void* table, int table_dtype,
                                          int64_t t_sbucket, int64_t t_shead, int h, bool has_bias, float tcol,
-                                         bool col_in_lanes, int padl, int qlen, int tid, int nthreads) {
+                                         bool col_in_lanes, int padl, int qlen, int tid, int nthreads,
+                                         int window = 0x7fffffff) {
     const float log2e = 1.4426950408889634f;
     // one evaluation per distance; the value goes to all four shifted copies
     for (int e0 = 0; e0 < qlen + 3; e0 += nthreads) {   // uniform trip count: the permute needs every lane
@@ -63,6 +64,7 @@ __device__ __forceinline__ void lut_fill(float* lut, const BucketSpec& bs, const
                 val = load_table(table, table_dtype, (int64_t)bk * t_sbucket + (int64_t)h * t_shead) * log2e;
         }
         if (CAUSAL && rel > 0) val = -INFINITY;
+        if (rel >= window || rel <= -window) val = -INFINITY;   // outside a sliding window folded into the LUT
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
             const int i = e - a;

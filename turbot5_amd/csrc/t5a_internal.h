@@ -24,7 +24,12 @@ struct BucketSpec {
 
 // kPacked: dense semantics per sequence of a packed batch (cu_seqlens); a separate instantiation, so that
 // the unpacked kernel carries none of its work-item search
-enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4 };
+// kLocal: sliding window of at most kMaxLutWindow, folded into the distance LUT; kLocalWide: wider windows, masked
+// per element at their edges
+enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLocalWide = 5 };
+// widest sliding window that is folded into the distance LUT (the LUT then spans 2 * (window + 96) distances;
+// 256 keeps it below 12 KB of LDS, so that two workgroups still share a compute unit)
+constexpr int kMaxLutWindow = 256;
 
 struct FwdParams {
     const void* q; const void* k; const void* v; void* o; float* lse;
@@ -42,6 +47,9 @@ struct FwdParams {
     const int32_t* plan; const int32_t* plan_counts; int plan_slots;
     int B, H, M, N;
     int tiles_per_seq;   // q tiles per (batch, head) when not packed
+    // sparse patterns with 16-bit inputs at head_dim 64 / 128: a work item is a run of run_len consecutive q tiles
+    // of one (batch, head) (the last run of a pair may be shorter); total_items = runs_per_seq * H * B
+    int run_len, runs_per_seq;
     int total_items;     // number of (q tile, head, batch) work items (upper bound when packed)
     // causal, unpacked, no key split (xcd_lo[8] > 0): items shrink with the tile index, so the list (pair-major,
     // longest tile first inside a (batch, head) pair) is cut into 8 slices of equal WORK, xcd_lo[x] .. xcd_lo[x+1]
