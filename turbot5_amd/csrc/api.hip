@@ -464,24 +464,48 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
             p.total_items = p.tiles_per_seq * a->H * a->B;
             return finish(launch_fwd(p, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, short)");
         }
-        // pass 1: rows >= G attend [global tokens | own block]
+        // rows >= G attend [global tokens | own block]; the G global queries attend every key with absolute positions
+        // (rel = j - i, no end alignment)
         const int nblk = (a->L + a->block_len - 1) / a->block_len;
         p.tiles_per_seq = nblk * ((a->block_len + 127) / 128);
         choose_runs(&p, kBlock, a->dtype, a->D);
+        const int G = a->aux < a->L ? a->aux : a->L;
+        const int64_t need = t5a_sparse_workspace_bytes(a->pattern, a->B, a->H, a->L, a->D, a->block_len, a->aux);
+        if (a->aux > 0 && a->workspace != nullptr && need > 0 && G <= 128) {
+            // one launch: the block items, then the global rows as key splits spread over the whole device; one merge
+            if (a->workspace_bytes < need)
+                return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes, %lld needed", (long long)a->workspace_bytes, (long long)need);
+            if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+            global_row_splits(a->B, a->H, a->L, &p.nsplit, &p.split_rows);
+            const int64_t rows = (int64_t)a->B * a->H * p.nsplit * G;
+            p.part_o = reinterpret_cast<float*>(a->workspace);
+            p.part_l = p.part_o + rows * a->D;
+            p.part_m = p.part_l + rows;
+            p.block_items = p.total_items;
+            const int64_t items = (int64_t)p.block_items + (int64_t)p.nsplit * a->H * a->B;
+            if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
+            p.total_items = (int)items;
+            rc = finish(launch_fwd(p, a->dtype, a->D, kBlock, false, s), "t5a_fwd_sparse(block + global rows as key splits)");
+            if (rc) return rc;
+            SplitKParams m;
+            memset(&m, 0, sizeof(m));
+            m.o = a->o; m.part_o = p.part_o; m.part_l = p.part_l; m.part_m = p.part_m;
+            m.o_sb = p.o_sb; m.o_sh = p.o_sh; m.o_sr = p.o_sr;
+            m.B = a->B; m.H = a->H; m.M = G; m.S = p.nsplit;
+            return finish(launch_splitk_merge(m, a->dtype, a->D, s), "t5a_fwd_sparse(block, merge)");
+        }
         rc = finish(launch_fwd(p, a->dtype, a->D, kBlock, false, s), "t5a_fwd_sparse(block)");
         if (rc || a->aux == 0) return rc;
-        // pass 2: the G global queries attend every key; positions are absolute, so M is
-        // clipped to G rows of the same tensors (rel = j - i, no end alignment)
+        // the G global queries as a pass of their own: M is clipped to G rows of the same tensors
         FwdParams g = p;
         g.run_len = 1;
-        g.M = a->aux < a->L ? a->aux : a->L;
+        g.M = G;
         g.N = a->L;
         g.tiles_per_seq = (g.M + 127) / 128;
         g.total_items = g.tiles_per_seq * a->H * a->B;
         g.align_end = 0;
-        const int64_t need = t5a_sparse_workspace_bytes(a->pattern, a->B, a->H, a->L, a->D, a->block_len, a->aux);
         if (a->workspace != nullptr && need > 0) {
-            // key splits over the whole device, then one merge
+            // (more than 128 global rows) key splits over the whole device in a second launch, then one merge
             if (a->workspace_bytes < need)
                 return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes, %lld needed", (long long)a->workspace_bytes, (long long)need);
             if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");

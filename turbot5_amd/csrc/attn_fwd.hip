@@ -313,6 +313,20 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const unsigned wi = (ga + (k - level * gx)) * tps + level;
         if (wi < lo || wi >= hi) return;
         w = (int)wi;
+    } else if (MODE == kBlock && p.nsplit > 1) {
+        // the key splits of the global rows are the longer items: they take the first workgroup ids, so that they
+        // start first and the block items fill in around them; the block items follow in per-XCD slices
+        const int n_split = p.total_items - p.block_items;
+        const int lead = (n_split + 7) & ~7;
+        if ((int)blockIdx.x < lead) {
+            if ((int)blockIdx.x >= n_split) return;
+            w = p.block_items + (int)blockIdx.x;
+        } else {
+            const int id = (int)blockIdx.x - lead;
+            const int per_xcd = (p.block_items + 7) >> 3;
+            w = (id & 7) * per_xcd + (id >> 3);
+            if (w >= p.block_items) return;
+        }
     } else {
         const int per_xcd = (p.total_items + 7) >> 3;
         w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
@@ -329,6 +343,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
+    bool gsplit = false;     // block pattern: this item is a key split of the global rows
     int n_side = p.n_side;   // side tokens of this item's sequence (transient-global)
     int64_t q_off, k_off, v_off, o_off, lse_off;
     if (MODE == kPacked) {
@@ -369,6 +384,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         unsigned bh = entry / (unsigned)p.tiles_per_seq;
         qt = (int)(entry - bh * (unsigned)p.tiles_per_seq);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
+        if (MODE == kBlock && p.nsplit > 1 && w >= p.block_items) {
+            // block pattern, behind the block items: key split `split` of the global rows of one (batch, head) --
+            // its first G rows attend all keys, standard bias; the partial results are merged by a second kernel
+            gsplit = true;
+            const unsigned gs = (unsigned)(w - p.block_items);
+            bh = gs / (unsigned)p.nsplit;
+            split = (int)(gs - bh * (unsigned)p.nsplit);
+            qt = 0;
+        }
         if (MODE == kDense && p.nsplit > 1) {
             const unsigned g = bh / (unsigned)p.nsplit;
             split = (int)(bh - g * (unsigned)p.nsplit);
@@ -390,7 +414,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
         v_off = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
         lse_off = (int64_t)b * p.lse_sb + (int64_t)h * p.lse_sh;
-        if (MODE == kDense && p.nsplit > 1) {   // this item sees only its slice of the keys
+        if ((MODE == kDense && p.nsplit > 1) || gsplit) {   // this item sees only its slice of the keys
+            if (gsplit) Mseq = min(p.aux, p.M);
             key0 = split * p.split_rows;
             Nseq = max(0, min(p.split_rows, p.N - key0));
             k_off += (int64_t)key0 * p.k_sr;
@@ -407,7 +432,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // query rows of the current q tile: [i0, row_end); rows below row_lo are computed but not stored
     int i0 = 0, row_end = 0, row_lo = 0, blk = 0;
     const int tpb = MODE == kBlock ? (p.block_len + BM - 1) / BM : 1;   // q tiles per block (block pattern)
-    if (MODE == kBlock) row_lo = p.aux;   // the first G rows belong to the global-query pass
+    if (MODE == kBlock && !gsplit) row_lo = p.aux;   // the first G rows belong to the key-split items / the global-query pass
     const int P = p.align_end ? Nseq - Mseq : -key0;   // query position minus row index, in this item's key numbering
 
     // ---------------------------------------------------------------- key segments
@@ -437,10 +462,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             seg_ksr[1] = (int)p.sk_sr * ES; seg_vsr[1] = (int)p.sv_sr * ES;
             seg_end[1] = n_side; seg_lend[1] = n_side; seg_kind[1] = 2;
         }
-    } else if (MODE == kBlock) {
+    } else if (MODE == kBlock && !gsplit) {
         nseg = 2;
         seg_end[0] = p.aux; seg_kind[0] = 1;
         seg_lend[1] = Nseq;
+    } else if (MODE == kBlock) {
+        seg_end[0] = Nseq;   // one segment: this split's keys, query i at position i (P = -key0)
     }
     // The part of the geometry that changes from one q tile to the next.  RUNS: every q tile of the run has the
     // same number of tiles per segment (seg_nt): the window starts where it starts even when that is before key 0,
@@ -448,7 +475,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // or masked.
     int seg_nt[2] = {0, 0};
     auto set_qtile = [&](int q_tile) {
-        if (MODE == kBlock) {
+        if (MODE == kBlock && !gsplit) {
             blk = q_tile / tpb;
             i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
             row_end = min(Mseq, (blk + 1) * p.block_len);
@@ -1320,10 +1347,10 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto store_rows = [&]() {
         const float l_tot = xhalf_sum(l_run + l_alt);
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        if (MODE == kDense && p.nsplit > 1) {
+        if ((MODE == kDense && p.nsplit > 1) || gsplit) {
             // partial result of a key split: normalised row in fp32, weight 1 (0: no visible key) and log-sum-exp
             if (row_ok) {
-                const int64_t prow = (((int64_t)b * p.H + h) * p.nsplit + split) * p.M + irow;
+                const int64_t prow = (((int64_t)b * p.H + h) * p.nsplit + split) * (gsplit ? Mseq : p.M) + irow;
                 float* orow = p.part_o + prow * D;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -1479,6 +1506,8 @@ static hipError_t launch_exact(const FwdParams& p, hipStream_t stream) {
         }
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
+    if (MODE == kBlock && p.nsplit > 1)
+        grid = (unsigned)(((p.total_items - p.block_items + 7) / 8) * 8 + ((p.block_items + 7) / 8) * 8);
     if (MODE == kPacked && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
     if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
         unsigned most = 0;

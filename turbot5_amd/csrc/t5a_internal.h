@@ -65,6 +65,9 @@ struct FwdParams {
     // key split (dense, unpacked, align_end == 0): split s of nsplit covers keys [s*split_rows, (s+1)*split_rows)
     // and writes its normalised partial rows, a 1/0 weight and its log-sum-exp to the workspace arrays
     int nsplit, split_rows;
+    // block pattern with key splits of its global rows in the same launch: the first block_items work items are the
+    // block items, then one item per (batch, head, split); the splits' rows are the first min(aux, M) rows
+    int block_items;
     float* part_o; float* part_l; float* part_m;   // (B,H,nsplit,M,D), (B,H,nsplit,M), (B,H,nsplit,M)
     BucketSpec bs;
 };
