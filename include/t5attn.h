@@ -91,7 +91,7 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 108
+#define T5A_ABI_VERSION 109
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -183,13 +183,20 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           reference computes them, attentions.py:722-732, :807-814).
  *   TGLOBAL block_len = window, aux = tokens per side token; side_k/side_v:
  *           (B,H,n_side,D) projected block aggregates, bias bucket(g - min(i/aux, n_side-1)).
- * seq_lens (optional, LOCAL and TGLOBAL): (B) int32 on the device, the number of valid tokens of each
- * right-padded sequence.  Keys at or past a sequence's length are not attended (the key half of the
- * reference's local mask, src/turbot5/model/utils.py:174-188); rows past the length are still
- * written (from the keys left in their window, zeros when there are none) and mean nothing.
- * TGLOBAL: a sequence of length n has n / aux side tokens, its tokens past the last full block
- * counting into the last one (utils.py:191-237 for a right-padded mask); side_k/side_v rows past
- * them are not read.
+ * seq_lens (optional): (B) int32 on the device, the number of valid tokens of each sequence; seq_starts
+ * (optional, LOCAL and TGLOBAL, with seq_lens): (B) int32, the row of its first token (a batch padded on the
+ * left; NULL = 0).  The tokens of sequence b are the rows [start, start + len); a token's position stays its
+ * row index, as in the reference.  Rows of padding tokens are still written and mean nothing.
+ *   LOCAL, TGLOBAL: keys outside the sequence's rows are not attended (the key half of the reference's local
+ *           mask, src/turbot5/model/utils.py:174-188).  TGLOBAL: the sequence has one side token per
+ *           aux-block END among its rows, (start + len) / aux - start / aux of them, a token's side token
+ *           being min(row / aux, count - 1) (utils.py:191-237 for one run of tokens); side_k/side_v rows
+ *           past them are not read.
+ *   BLOCK   (right padding only) the reference's additive mask as it lays it out
+ *           (src/turbot5/model/attentions.py:722-732): in block b, list column c < block_len of
+ *           [G global tokens | own block] is masked iff token b * block_len + c is padding, the last G
+ *           columns never (always in block 0); the first G rows attend every key, padding included
+ *           (:788-800).
  * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
  * the G global rows, which attend all L keys, are computed as key splits spread over the whole
  * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
@@ -206,6 +213,7 @@ typedef struct t5a_sparse_args {
     float sm_scale; int32_t exact_scores;
     t5a_bias bias;
     const int32_t* seq_lens;
+    const int32_t* seq_starts;
 } t5a_sparse_args;
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux);
 int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);
@@ -265,9 +273,11 @@ int t5a_fwd_splitk_static(const t5a_splitk_args* args, t5a_stream_t stream);
  * weight's type when that is 16 bit, else fp32 (torch type promotion of the reference code).
  * Arithmetic as the reference's eager path: fp32 variance and scaling, the scaled value rounded to
  * a 16-bit weight's type before the product; block sums are rounded to the input type first.
- * seq_lens (optional, not together with residual): (batches) int32 on the device, valid rows of each right-padded
- * batch element: it has seq_len / group groups (its rows past the last full group join that group,
- * padding rows are left out); output rows past them are zero.
+ * seq_lens / seq_starts (optional, not together with residual): (batches) int32 on the device, the rows
+ * [start, start + len) of each batch element are its tokens (seq_starts NULL = 0): it has one group per group END
+ * among them, (start + len) / group - start / group, group g taking its tokens of rows [g * group,
+ * (g + 1) * group) and the last group every token from there on; groups without a token and output rows past
+ * the groups are zero.
  * residual (optional, group == 1 only): rows of x's type and shape with row stride
  * residual_row_stride; the kernel normalises x + residual (rounded to x's type, as torch's add leaves
  * it) and also writes that sum to sum_out (x's type, rows contiguous like y, 16-byte aligned; must
@@ -282,6 +292,7 @@ typedef struct t5a_rmsnorm_args {
     int32_t reserved;
     const void* residual; void* sum_out; int64_t residual_row_stride;
     const int32_t* seq_lens;
+    const int32_t* seq_starts;   /* optional, with seq_lens: first valid row of each batch element (NULL = 0) */
 } t5a_rmsnorm_args;
 int t5a_rmsnorm(const t5a_rmsnorm_args* args, t5a_stream_t stream);
 

@@ -58,7 +58,7 @@ def basic_self_attention(sd: SD, prefix: str, cfg, hidden: torch.Tensor, table: 
     elif attention_type == "local":
         out = O.local_attention_blocked(q, k, v, table, cfg.sliding_window, key_mask, nb, md)
     elif attention_type == "block":
-        out = O.block_attention_blocked(q, k, v, table, cfg.sliding_window, cfg.global_block_size, None, nb, md)
+        out = O.block_attention_blocked(q, k, v, table, cfg.sliding_window, cfg.global_block_size, key_mask, nb, md)
     elif attention_type == "transient-global":
         gbs = cfg.global_block_size
         side = tglobal_side_inputs(hidden, gbs, sd[prefix + "global_input_layer_norm.weight"], cfg.layer_norm_epsilon,

@@ -63,10 +63,11 @@ def test_attention_module_output_tuple(gpu_device):
         assert out2[0].shape == (2, 96, 128)
     mask = torch.ones(2, 96, device=gpu_device)
     mask[1, 50:] = 0
-    with pytest.raises(NotImplementedError):         # right padding: local and transient-global only
-        T5ATTENTION_TYPES["block"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
     mask[0, :3] = 0
-    for name in ("local", "transient-global"):       # left padding
+    with pytest.raises(NotImplementedError):         # left padding: local and transient-global only
+        T5ATTENTION_TYPES["block"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
+    mask[1, 20:30] = 0
+    for name in ("local", "block", "transient-global"):       # holes
         with pytest.raises(NotImplementedError):
             T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
 
@@ -287,10 +288,19 @@ def test_local_encoder_with_right_padding(gpu_device):
         got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
     valid = mask.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+    # padding on the left, and on both sides: a first row and a length per sequence; positions stay row indices
     left = torch.ones(3, 256)
     left[1, :10] = 0
+    left[2, :77] = 0
+    left[2, 250:] = 0
+    want = OM.encoder_forward(sd, cfg, ids, left, attention_type="local")
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), left.to(gpu_device)).cpu()
+    assert (got[left.bool()] - want[left.bool()]).abs().max().item() <= 2e-3
+    holes = torch.ones(3, 256)
+    holes[1, 40:50] = 0
     with pytest.raises(NotImplementedError), torch.no_grad():
-        m(ids.to(gpu_device), left.to(gpu_device))
+        m(ids.to(gpu_device), holes.to(gpu_device))
 
 
 def test_transient_global_encoder_with_right_padding(gpu_device):
@@ -307,6 +317,40 @@ def test_transient_global_encoder_with_right_padding(gpu_device):
         got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
     valid = mask.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+    # padding on the left and on both sides: the reference's block ids for such rows (side tokens before the first
+    # token are empty, the last one takes every token from its first row on), first rows inside a side block
+    left = torch.ones(3, 256)
+    left[0, :19] = 0
+    left[1, :64] = 0
+    left[1, 201:] = 0
+    left[2, :5] = 0
+    left[2, 9:] = 0                  # four tokens: no side token at all
+    want = OM.encoder_forward(sd, cfg, ids, left, attention_type="transient-global")
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), left.to(gpu_device)).cpu()
+    assert (got[left.bool()] - want[left.bool()]).abs().max().item() <= 2e-3
+
+
+def test_block_encoder_with_right_padding(gpu_device):
+    """T5BlockAttention on right-padded batches: the reference's additive mask as it lies over the key list
+    [global tokens | own block] (its layout quirk included), global rows seeing every key."""
+    cfg, m, sd = make(dict(SMALL, attention_type="block", sliding_window=64, global_block_size=16))
+    ids = torch.randint(0, 200, (4, 256), generator=torch.Generator().manual_seed(11))
+    mask = torch.ones(4, 256)
+    mask[0, 200:] = 0                # inside the last block, past its first 16 columns
+    mask[1, 70:] = 0                 # inside the second block, within its first 16 columns
+    mask[2, 30:] = 0                 # inside block 0
+    mask[3, 128:] = 0                # exactly at a block boundary
+    want = OM.encoder_forward(sd, cfg, ids, mask, attention_type="block")
+    m = m.to(gpu_device)
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
+    valid = mask.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
+    left = torch.ones(4, 256)
+    left[1, :10] = 0
+    with pytest.raises(NotImplementedError), torch.no_grad():
+        m(ids.to(gpu_device), left.to(gpu_device))
 
 
 @pytest.mark.parametrize("attention_dtype", [None, torch.bfloat16])

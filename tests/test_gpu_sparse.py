@@ -155,12 +155,14 @@ def test_local_with_sequence_lengths(gpu_device, dtype, L, Bl, lens):
     assert torch.equal(a, b_)
 
 
-def test_sequence_lengths_are_not_for_the_block_pattern(gpu_device):
+def test_sequence_length_arguments_are_checked(gpu_device):
     from turbot5_amd import ops
     q = torch.zeros(1, 1, 128, 64, device=gpu_device, dtype=torch.bfloat16)
     lens = torch.tensor([100], dtype=torch.int32, device=gpu_device)
-    with pytest.raises(ValueError):
-        ops._sparse(ops.L.PATTERN_BLOCK, q, q, q, None, 64, 16, seq_lens=lens)
+    with pytest.raises(ValueError):          # first rows are for the windowed patterns
+        ops._sparse(ops.L.PATTERN_BLOCK, q, q, q, None, 64, 16, seq_lens=lens, seq_starts=lens)
+    with pytest.raises(ValueError):          # ... and need lengths
+        ops.local_attention_with_fusing_bias(q, q, q, None, 64, seq_starts=lens)
     with pytest.raises(ValueError):
         ops.local_attention_with_fusing_bias(q, q, q, None, 64, seq_lens=lens.long())
 
@@ -244,3 +246,48 @@ def test_local_with_runs_of_q_tiles(gpu_device, monkeypatch, run_len, L, Bl):
         wb = O.basic_attention(q[b:b + 1, :, :n].float(), k[b:b + 1, :, :n].float(), v[b:b + 1, :, :n].float(),
                                bias[:, :, :n, :n])
         assert (out_l[b:b + 1, :, :n] - wb).abs().max().item() <= 2e-2, b
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,G", [(1024, 128, 64), (512, 64, 64), (768, 256, 32), (640, 128, 0)])
+def test_block_with_right_padded_sequences(gpu_device, dtype, L, Bl, G):
+    """Per-sequence lengths in the block pattern against the oracle's mask path (pinned by vectors from the
+    reference module): lengths inside block 0, inside a later block on either side of its first G columns, at a
+    block boundary, and a full sequence; with and without key splits for the global rows."""
+    from turbot5_amd.ops import block_attention_with_fusing_bias
+    H, D = 3, 64
+    lens = [L, Bl // 2, Bl + G // 2 + 1, 2 * Bl + G + 5, 3 * Bl, L - 1]
+    B = len(lens)
+    q, k, v = (rnd(B, H, L, D, seed=400 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=403, scale=1.0)
+    mask = (torch.arange(L)[None, :] < torch.tensor(lens)[:, None]).float()
+    want = O.block_attention_blocked(q, k, v, table, Bl, G, mask)
+    tl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    dev = [t.to(gpu_device) for t in (q, k, v, table)]
+    for splits in (True, False):
+        out = block_attention_with_fusing_bias(*dev, Bl, G, seq_lens=tl, key_splits=splits).float().cpu()
+        for b, n in enumerate(lens):
+            err = (out[b, :, :n] - want[b, :, :n]).abs().max().item()
+            assert err <= TOL[dtype], (b, n, splits, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl", [(1024, 128), (512, 64), (1536, 512)])
+def test_local_with_padding_on_either_side(gpu_device, dtype, L, Bl):
+    from turbot5_amd.ops import local_attention_with_fusing_bias
+    H, D = 3, 64
+    spans = [(0, L), (37, L - 37), (Bl + 3, 2 * Bl), (L - 70, 70), (5, 1), (0, 0)]
+    B = len(spans)
+    q, k, v = (rnd(B, H, L, D, seed=410 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=413, scale=1.0)
+    pos = torch.arange(L)[None, :]
+    st, ln = torch.tensor([s for s, _ in spans])[:, None], torch.tensor([n for _, n in spans])[:, None]
+    mask = ((pos >= st) & (pos < st + ln)).float()
+    want = O.local_attention_blocked(q, k, v, table, Bl, mask)
+    out = local_attention_with_fusing_bias(
+        *(t.to(gpu_device) for t in (q, k, v, table)), Bl,
+        seq_lens=ln[:, 0].to(torch.int32).to(gpu_device), seq_starts=st[:, 0].to(torch.int32).to(gpu_device)).float().cpu()
+    valid = mask.bool()
+    assert torch.isfinite(out[valid[:, None, :].expand(B, H, L)]).all()
+    err = (out - want).abs()[valid[:, None, :, None].expand(B, H, L, D)].max().item()
+    assert err <= TOL[dtype], err

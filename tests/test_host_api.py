@@ -35,9 +35,9 @@ def test_struct_sizes_follow_the_header(lib):
     assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
-    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 8
+    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 2 * 8
     assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4 + 2 * 8
-    assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 4 * 8
+    assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 5 * 8
 
 
 @pytest.mark.parametrize("bidirectional", [True, False])
@@ -226,16 +226,19 @@ def test_mask_info_is_not_inherited_by_another_tensor():
 
 
 def test_sequence_length_arguments_are_checked_without_gpu(lib):
-    """seq_lens belongs to the windowed patterns and to the grouped norm; the checks come before any launch"""
+    """seq_starts belongs to the windowed patterns and needs seq_lens; the checks come before any launch"""
     handle = lib.load()
     s = lib.T5ASparseArgs()
     s.dtype, s.B, s.H, s.L, s.D, s.pattern, s.block_len, s.aux = 0, 1, 1, 256, 64, 2, 64, 16    # block pattern
     s.q = s.k = s.v = s.o = 0x1000
     for name in ("q_strides", "k_strides", "v_strides", "o_strides"):
         setattr(s, name, (C.c_int64 * 3)(256 * 64, 256 * 64, 64))
-    s.seq_lens = 0x3000
-    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7
-    assert b"seq_lens" in handle.t5a_last_error()
+    s.seq_lens, s.seq_starts = 0x3000, 0x3100
+    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7           # first rows: windowed patterns only
+    assert b"seq_starts" in handle.t5a_last_error()
+    s.pattern, s.aux, s.seq_lens = 1, 0, None
+    assert handle.t5a_fwd_sparse(C.byref(s), None) == -7           # first rows without lengths
+    assert b"seq_starts" in handle.t5a_last_error()
     r = lib.T5ARmsNormArgs()
     r.x, r.weight, r.y = 0x1000, 0x2000, 0x4000
     r.x_strides = (C.c_int64 * 2)(0, 64)
@@ -246,6 +249,10 @@ def test_sequence_length_arguments_are_checked_without_gpu(lib):
     assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # lengths and a residual do not go together
     assert b"seq_lens" in handle.t5a_last_error()
     r.seq_lens = None
+    r.seq_starts = 0x3100
+    r.residual = None
+    assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # first rows without lengths
+    r.seq_starts, r.residual = None, 0x5000
     r.group, r.rows_per_batch = 2, 8
     assert handle.t5a_rmsnorm(C.byref(r), None) == -4          # a residual needs group == 1
     r.group, r.sum_out = 1, 0x1000

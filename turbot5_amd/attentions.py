@@ -13,8 +13,8 @@ libt5attn.so; there is no torch fallback in this package.
 Differences from the reference, all on purpose:
 * every module hands the (num_buckets, H) TABLE on as ``position_bias`` (the reference does so
   for 'flash' only; the sparse modules materialise a bias tensor), and never builds an L x L bias;
-* the sparse modules accept only all-ones attention masks (what ``T5Stack`` supplies when the
-  caller gives none); other masks raise ``NotImplementedError``;
+* the sparse modules take attention masks whose rows are one run of valid tokens (all ones, right padding,
+  and for local / transient-global also left padding); masks with holes raise ``NotImplementedError``;
 * transient-global returns the head-correct layout (the reference's ``unshape`` omits the
   head transpose, attentions.py:951-953);
 * ``layer_head_mask`` and ``output_attentions`` are not available on fused paths.
@@ -42,13 +42,14 @@ class T5LayerNorm(nn.Module):
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(dim))
 
-    def forward(self, x: torch.Tensor, group: int = 1, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, group: int = 1, seq_lens: Optional[torch.Tensor] = None,
+                seq_starts: Optional[torch.Tensor] = None) -> torch.Tensor:
         """On a ROCm device: the fused HIP kernel (the reference switches to its Triton kernel there,
         modules.py:61-66).  Host tensors take the reference's eager formula (modules.py:51-59).
         ``group`` > 1 norms the sums of ``group`` consecutive rows of each sequence (side tokens)."""
         if x.is_cuda:
             from .ops import rms_norm
-            return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens)
+            return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens, seq_starts=seq_starts)
         if group > 1:
             B, L, d = x.shape
             n = L // group
@@ -351,9 +352,10 @@ class T5FlashAttention(_T5AttentionBase):
 
 
 class _SparseBase(_T5AttentionBase):
-    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                    right_padding_ok=False):
-        """Returns the (B,) int32 lengths of a right-padded batch when the pattern supports them, else None."""
+    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions, left_padding_ok=True):
+        """-> (lengths, first rows): (B,) int32 device tensors for a batch whose rows are each ONE run of valid
+        tokens (padding on the right, and on the left where the pattern takes it); (None, None) for all ones.
+        First rows are None for right padding."""
         if past_key_value is not None:
             warnings.warn('Currently, passing past key value states is not supported.')
         if use_cache is not None:
@@ -362,13 +364,22 @@ class _SparseBase(_T5AttentionBase):
         if mask is not None:
             all_ones, unpad = _mask_info(mask)
             if not all_ones:
-                if right_padding_ok and unpad[0] == "lens" and unpad[2].get("right_padded"):
-                    return unpad[1][0]
+                if unpad[0] == "lens":
+                    plans = unpad[2]
+                    if plans.get("right_padded"):
+                        return unpad[1][0], None
+                    if left_padding_ok:
+                        starts = plans.get("starts")
+                        if starts is None:   # first row of each sequence, from the start rows of the flat (B*L) layout
+                            B, L = mask.shape
+                            starts = plans["starts"] = (unpad[1][1][:B] - torch.arange(
+                                B, device=mask.device, dtype=torch.int32) * L).contiguous()
+                        return unpad[1][0], starts
                 raise NotImplementedError(
-                    f"{type(self).__name__} runs as tile skipping for all-ones attention masks"
-                    + (" and right-padded batches" if right_padding_ok else "")
-                    + " only; use attention_type='flash' for other padded batches")
-        return None
+                    f"{type(self).__name__} runs as tile skipping for attention masks whose rows are one run of valid "
+                    "tokens (padding on the right" + (" or on the left" if left_padding_ok else "")
+                    + "); use attention_type='flash' for masks with holes")
+        return None, None
 
     def _qkv(self, hidden_states):
         batch_size = hidden_states.shape[0]
@@ -392,15 +403,14 @@ class T5LocalAttention(_SparseBase):
                 use_cache=None, output_attentions=False):
         # right-padded batches: the keys of a sequence end at its length (the key half of the reference's
         # local mask, utils.py:174-188); outputs at padded positions mean nothing, as in the reference
-        seq_lens = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                                    right_padding_ok=True)
+        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
         # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
         block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.local_attention_with_fusing_bias(
             q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance, seq_lens=seq_lens,
+            self.relative_attention_max_distance, seq_lens=seq_lens, seq_starts=seq_starts,
             exact_scores=self._exact)
         return self._finish(out, hidden_states, table)
 
@@ -415,12 +425,16 @@ class T5BlockAttention(_SparseBase):
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
-        self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        # right-padded batches: the reference's additive mask over its key list (attentions.py:722-732)
+        seq_lens, _ = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
+                                       left_padding_ok=False)
+        if seq_lens is not None and hidden_states.shape[1] < self.block_len:
+            raise NotImplementedError("T5BlockAttention: padded batches shorter than one block are not supported")
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
         out = ops.block_attention_with_fusing_bias(
             q, k, v, table, self.block_len, self.n_global_tokens, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance, exact_scores=self._exact)
+            self.relative_attention_max_distance, exact_scores=self._exact, seq_lens=seq_lens)
         return self._finish(out, hidden_states, table)
 
 
@@ -437,7 +451,8 @@ class T5TransientGlobalAttention(_SparseBase):
             self.global_relative_attention_bias = nn.Embedding(self.relative_attention_num_buckets, self.n_heads)
         self.global_input_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
-    def side_inputs(self, hidden_states: torch.Tensor, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def side_inputs(self, hidden_states: torch.Tensor, seq_lens: Optional[torch.Tensor] = None,
+                    seq_starts: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Normalised block sums, (B, L // global_block_size, d_model); trailing tokens that do not fill
         a block join the last one (utils.py:206-212, :249-258; attentions.py:959-966).  With ``seq_lens``
         each right-padded sequence counts its valid tokens only."""
@@ -446,17 +461,17 @@ class T5TransientGlobalAttention(_SparseBase):
         n_side = L // gbs
         if n_side == 0:
             return hidden_states.new_zeros(B, 0, d)
-        return self.global_input_layer_norm(hidden_states, group=gbs, seq_lens=seq_lens)   # block sums and norm in one kernel
+        # block sums and norm in one kernel
+        return self.global_input_layer_norm(hidden_states, group=gbs, seq_lens=seq_lens, seq_starts=seq_starts)
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
         # right-padded batches: per-sequence key limit and side-token count in the kernels (utils.py:174-237)
-        seq_lens = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                                    right_padding_ok=True)
+        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
         batch_size = hidden_states.shape[0]
         adt = self._attn_dtype(hidden_states)
         q, k, v = self._qkv(hidden_states)
-        side = self.side_inputs(hidden_states, seq_lens)
+        side = self.side_inputs(hidden_states, seq_lens, seq_starts)
         side_k = self._shape(self.k(side), batch_size).to(adt)
         side_v = self._shape(self.v(side), batch_size).to(adt)
         table = self._table(position_bias)
@@ -464,7 +479,7 @@ class T5TransientGlobalAttention(_SparseBase):
         out = ops.transient_global_attention_with_fusing_bias(
             q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
             self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens,
-            exact_scores=self._exact)
+            seq_starts=seq_starts, exact_scores=self._exact)
         return self._finish(out, hidden_states, table)
 
 

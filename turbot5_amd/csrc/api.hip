@@ -446,10 +446,10 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.sk_sb = a->side_k_strides[0]; p.sk_sh = a->side_k_strides[1]; p.sk_sr = a->side_k_strides[2];
     p.sv_sb = a->side_v_strides[0]; p.sv_sh = a->side_v_strides[1]; p.sv_sr = a->side_v_strides[2];
     p.B = a->B; p.H = a->H; p.M = a->L; p.N = a->L;
-    if (a->seq_lens != nullptr) {
-        if (a->pattern == T5A_PATTERN_BLOCK) return fail(T5A_ERR_PATTERN, "seq_lens is supported by the local and transient-global patterns only");
-        p.len_k = a->seq_lens;
-    }
+    if (a->seq_starts != nullptr && (a->seq_lens == nullptr || a->pattern == T5A_PATTERN_BLOCK))
+        return fail(T5A_ERR_PATTERN, "seq_starts needs seq_lens and the local or transient-global pattern");
+    p.len_k = a->seq_lens;
+    p.start_k = a->seq_starts;
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
     p.c1 = a->sm_scale * kLog2e;
     p.exact_scale = a->exact_scores != 0;
@@ -462,6 +462,8 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
             // shorter than one block: the reference degenerates to full attention (attentions.py:752, :691)
             p.tiles_per_seq = (a->L + 127) / 128;
             p.total_items = p.tiles_per_seq * a->H * a->B;
+            if (a->seq_lens != nullptr)
+                return fail(T5A_ERR_PATTERN, "block pattern: seq_lens with a sequence shorter than one block is not supported");
             return finish(launch_fwd(p, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, short)");
         }
         // rows >= G attend [global tokens | own block]; the G global queries attend every key with absolute positions
@@ -499,6 +501,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         // the G global queries as a pass of their own: M is clipped to G rows of the same tensors
         FwdParams g = p;
         g.run_len = 1;
+        g.len_k = nullptr;
         g.M = G;
         g.N = a->L;
         g.tiles_per_seq = (g.M + 127) / 128;
@@ -653,6 +656,9 @@ int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
     if (a->seq_lens != nullptr) {
         if (a->residual != nullptr) return fail(T5A_ERR_SHAPE, "seq_lens and residual cannot be combined");
         p.lens = a->seq_lens;
+        p.starts = a->seq_starts;
+    } else if (a->seq_starts != nullptr) {
+        return fail(T5A_ERR_SHAPE, "seq_starts needs seq_lens");
     }
     p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;
     p.out_per_batch = out_per_batch;

@@ -344,6 +344,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     bool gsplit = false;     // block pattern: this item is a key split of the global rows
+    int key_lo = 0;          // windowed patterns: first key of the sequence (a batch padded on the left)
+    int n_valid = 0x7fffffff;   // block pattern: valid tokens of a right-padded sequence
     int n_side = p.n_side;   // side tokens of this item's sequence (transient-global)
     int64_t q_off, k_off, v_off, o_off, lse_off;
     if (MODE == kPacked) {
@@ -406,9 +408,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         // the row indices, so nothing else changes (rows past the length see what is left of their window).
         // Its side tokens are the full blocks of that length, the rest of its tokens joining the last one.
         if ((LOCAL || MODE == kTGlobal) && p.len_k != nullptr) {
-            Nseq = max(0, min(p.N, p.len_k[b]));
-            if (MODE == kTGlobal) n_side = min(p.n_side, Nseq / p.aux);
+            // the sequence's tokens are the rows [key_lo, Nseq); a token's position stays its row index
+            key_lo = p.start_k != nullptr ? max(0, min(p.N, p.start_k[b])) : 0;
+            Nseq = max(key_lo, min(p.N, key_lo + max(0, p.len_k[b])));
+            // side tokens: one per block END among the tokens; a token's side token is min(row / aux, count - 1)
+            // (what the reference's block ids come to for one run of tokens, src/turbot5/model/utils.py:191-237)
+            if (MODE == kTGlobal) n_side = min(p.n_side, Nseq / p.aux - key_lo / p.aux);
         }
+        if (MODE == kBlock && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -474,13 +481,28 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // and a block's segment spans a whole block; tiles outside the keys that exist read as zeros and are skipped
     // or masked.
     int seg_nt[2] = {0, 0};
+    int hole_lo = 0, hole_span = 0;   // block pattern, padded sequence: own-block keys [hole_lo, hole_lo + hole_span) are masked
     auto set_qtile = [&](int q_tile) {
         if (MODE == kBlock && !gsplit) {
             blk = q_tile / tpb;
             i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
             row_end = min(Mseq, (blk + 1) * p.block_len);
             seg_start[1] = blk * p.block_len;
-            seg_end[1] = blk == 0 ? p.block_len - p.aux : (blk + 1) * p.block_len;
+            // The reference lays its additive padding mask out as [own block | global tokens] over keys that are
+            // laid out [global tokens | own block] (src/turbot5/model/attentions.py:722-732 against :807-814): list
+            // column c < block_len is masked iff token blk * block_len + c is padding, the last G columns never are
+            // (except in block 0, where they always are).  valid = how many of the first block_len list columns stay.
+            const int valid = max(0, min(p.block_len, n_valid - blk * p.block_len));
+            seg_end[0] = min(p.aux, valid);
+            const int head = max(valid - p.aux, 0);           // own-block keys before the masked range
+            if (blk == 0) {
+                seg_end[1] = min(p.block_len - p.aux, head);
+                hole_span = 0;
+            } else {
+                seg_end[1] = (blk + 1) * p.block_len;
+                hole_lo = blk * p.block_len + head;
+                hole_span = max(0, p.block_len - p.aux - head);
+            }
         } else {
             i0 = q_tile * BM;
             row_end = Mseq;
@@ -488,7 +510,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (DENSE) {
             seg_end[0] = CAUSAL ? max(0, min(Nseq, i0 + BM + P)) : Nseq;
         } else if (LOCAL || MODE == kTGlobal) {
-            seg_start[0] = RUNS ? i0 - p.block_len + 1 : max(0, i0 - p.block_len + 1);
+            seg_start[0] = RUNS ? i0 - p.block_len + 1 : max(key_lo, i0 - p.block_len + 1);
             seg_end[0] = min(Nseq, min(i0 + BM, Mseq) - 1 + p.block_len);
         }
     };
@@ -946,10 +968,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const int s_end = c.sg ? seg_end[1] : seg_end[0];
         c.need_mask = c.j0 + BN > s_end;
         if constexpr (RUNS) {   // tiles before key 0 or past the end of the segment exist here (same count for every q tile)
-            c.skip = c.skip || c.j0 >= s_end || c.j0 + BN <= 0;
-            c.need_mask = c.need_mask || c.j0 < 0;
+            c.skip = c.skip || c.j0 >= s_end || c.j0 + BN <= key_lo;
+            c.need_mask = c.need_mask || c.j0 < key_lo;
         }
         if (win && !win_lut) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
+        if (MODE == kBlock && c.sg == 1 && hole_span > 0)
+            c.need_mask = c.need_mask || (c.j0 < hole_lo + hole_span && c.j0 + BN > hole_lo);
         c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
         if constexpr (win_lut) c.side = 0;
         return c;
@@ -1110,16 +1134,22 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0 && !win_lut;
             const int qpos = lane_qpos(c.sg);
             // this lane's row sees the keys [lo, hi): one subtraction and one unsigned compare per element
-            const int lo = win ? max(0, qpos - p.block_len + 1) : 0;
+            const int seg_lo = (c.sg == 0 && (LOCAL || MODE == kTGlobal)) ? key_lo : 0;   // first key of the sequence
+            const int lo = win ? max(seg_lo, qpos - p.block_len + 1) : seg_lo;
             const int hi = win ? min(s_end, qpos + p.block_len) : s_end;
             const unsigned span = (unsigned)max(hi - lo, 0);
             const int jl = c.j0 + 4 * hh - lo;
+            // block pattern on a padded sequence: a range of the own block's keys that the rows do not see
+            const unsigned hspan = (MODE == kBlock && c.sg == 1) ? (unsigned)hole_span : 0u;
+            const int jh = c.j0 + 4 * hh - hole_lo;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const unsigned j = (unsigned)(jl + 32 * nt + 8 * (r >> 2) + (r & 3));
-                    st[nt][r] = j < span ? st[nt][r] : -INFINITY;
+                    const int off = 32 * nt + 8 * (r >> 2) + (r & 3);
+                    bool keep = (unsigned)(jl + off) < span;
+                    if (MODE == kBlock) keep = keep && !((unsigned)(jh + off) < hspan);
+                    st[nt][r] = keep ? st[nt][r] : -INFINITY;
                 }
         }
         // st already holds (score - m_run)
@@ -1256,7 +1286,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     f32x16 sta[NT], stb[NT];
     fill_classes();
     TileClass tc = classify(0);
-    const bool first_interior = LOCAL && seg_start[0] >= 0 && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+    const bool first_interior = LOCAL && seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
     if constexpr (QDMA) {
         // K0 and V0 landed before the barrier that published the LUT
     } else {
@@ -1453,7 +1483,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             for (int r = 0; r < 16; ++r) cm[r] = 0.f;
             // away from the ends of the sequence every q tile of the local pattern has the same classes
             const bool was_interior = interior;
-            interior = LOCAL && seg_start[0] >= 0 && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+            interior = LOCAL && seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
             if (!(interior && was_interior)) fill_classes();
             tc = classify(0);
             if (tc.side != 0) refill_cm(tc.side);

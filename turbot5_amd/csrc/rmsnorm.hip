@@ -45,19 +45,22 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     if (row >= p.out_rows) return;
     const int64_t b = row / p.out_per_batch;
     const int g = (int)(row - b * p.out_per_batch);
-    const int first = g * p.group;
-    // with per-sequence lengths a sequence has len / group groups, the rest of its rows joining the last
-    // one; output rows past them are zero
-    const int rows_b = p.lens ? max(0, min(p.rows_per_batch, p.lens[b])) : p.rows_per_batch;
-    const int groups_b = p.lens ? rows_b / p.group : p.out_per_batch;
-    const int count = g == groups_b - 1 ? rows_b - first : p.group;
+    // With per-sequence lengths (and first rows) a sequence is the rows [start, end).  It has one group per group END
+    // among its rows, group g taking its rows of [g * group, (g + 1) * group) and the last group every row from
+    // there on (the reference's block ids for one run of tokens: min(row / group, groups - 1),
+    // src/turbot5/model/utils.py:191-237); groups without a row and output rows past the groups are zero.
+    const int start_b = p.starts ? max(0, min(p.rows_per_batch, p.starts[b])) : 0;
+    const int end_b = p.lens ? min(p.rows_per_batch, start_b + max(0, p.lens[b])) : p.rows_per_batch;
+    const int groups_b = p.lens ? end_b / p.group - start_b / p.group : p.out_per_batch;
+    const int first = max(start_b, g * p.group);
+    const int count = (g == groups_b - 1 ? end_b : min((g + 1) * p.group, end_b)) - first;
     const TX* x = reinterpret_cast<const TX*>(p.x) + b * p.x_batch_stride + (int64_t)first * p.x_row_stride;
     const TX* res = p.residual ? reinterpret_cast<const TX*>(p.residual) + row * p.residual_row_stride : nullptr;
     TX* sum = res ? reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride : nullptr;
     const TW* w = reinterpret_cast<const TW*>(p.weight);
     TY* y = reinterpret_cast<TY*>(p.y) + row * p.y_row_stride;
     const int nch = p.dim / VEC;
-    if (g >= groups_b) {
+    if (g >= groups_b || count <= 0) {
         Vec<TY, VEC> zero;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) zero.v[i] = Cvt<TY>::down(0.f);

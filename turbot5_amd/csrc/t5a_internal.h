@@ -43,6 +43,7 @@ struct FwdParams {
     int64_t lse_sb, lse_sh, lse_sr;
     const int32_t* cu_q; const int32_t* cu_k;   // non-null: packed variable-length batch
     const int32_t* len_q; const int32_t* len_k; // optional lengths (rows between cu[b]+len[b] and cu[b+1] are padding)
+    const int32_t* start_k;                     // sparse patterns, optional: first token of each sequence (left padding)
     // packed batch with a launch plan (plan.hip): workgroup 8 k + x runs the item in plan[x][k]
     const int32_t* plan; const int32_t* plan_counts; int plan_slots;
     int B, H, M, N;
@@ -120,6 +121,7 @@ struct RmsParams {
     const void* x; const void* weight; void* y;
     const void* residual; void* sum_out;                  // optional: normalise x + residual, write the sum (input type)
     const int* lens;                                      // optional (group > 1): valid rows per batch element
+    const int* starts;                                    // optional, with lens: first valid row per batch element
     int64_t residual_row_stride;
     int64_t x_batch_stride, x_row_stride, y_row_stride;   // elements
     int64_t out_rows;        // batches * out_per_batch

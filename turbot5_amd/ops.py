@@ -318,14 +318,14 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
 
 
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
-            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None):
+            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None, seq_starts=None):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
-    if seq_lens is not None:
-        if pattern == L.PATTERN_BLOCK:
-            raise ValueError("seq_lens is supported by the local and transient-global patterns only")
-        if seq_lens.dtype != torch.int32 or seq_lens.shape != (B,) or seq_lens.device != q.device or not seq_lens.is_contiguous():
-            raise ValueError("seq_lens must be a contiguous int32 tensor of shape (B,) on the device of q")
+    for name, t in (("seq_lens", seq_lens), ("seq_starts", seq_starts)):
+        if t is not None and (t.dtype != torch.int32 or t.shape != (B,) or t.device != q.device or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous int32 tensor of shape (B,) on the device of q")
+    if seq_starts is not None and (seq_lens is None or pattern == L.PATTERN_BLOCK):
+        raise ValueError("seq_starts needs seq_lens and the local or transient-global pattern")
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("sparse self-attention needs q, k, v of one shape")
     q_, k_, v_ = (_kernel_ready(t) for t in (q, k, v))
@@ -350,6 +350,8 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     a.exact_scores = _exact(exact_scores)
     if seq_lens is not None:
         a.seq_lens = seq_lens.data_ptr()
+    if seq_starts is not None:
+        a.seq_starts = seq_starts.data_ptr()
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
     lib = L.load()
     ws_bytes = lib.t5a_sparse_workspace_bytes(pattern, B, H, Lq, D, int(block_len), int(aux))
@@ -364,41 +366,46 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
 
 
 def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                     seq_lens=None, exact_scores=None):
+                                     seq_lens=None, exact_scores=None, seq_starts=None):
     """Sliding-window self-attention: key j visible to query i iff |j-i| < block_len, bias bucket(j-i).
 
     The op of T5LocalAttention (src/turbot5/model/attentions.py:583-638) without
     blocking, K/V triplication or a bias tensor.  q,k,v (B,H,L,D).
-    ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; keys past a sequence's length are
-    not attended (the mask of src/turbot5/model/utils.py:174-188 for its valid query rows)."""
+    ``seq_lens`` / ``seq_starts`` (B,) int32: the tokens of sequence b are the rows [start, start + len) (start
+    defaults to 0: right padding); keys outside them are not attended (the mask of
+    src/turbot5/model/utils.py:174-188 for the sequence's own rows), positions stay the row indices."""
     return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE,
-                   seq_lens=seq_lens, exact_scores=exact_scores)
+                   seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts)
 
 
 def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
-                                     MAX_DISTANCE=128, key_splits=True, exact_scores=None):
+                                     MAX_DISTANCE=128, key_splits=True, exact_scores=None, seq_lens=None):
     """Block attention with ``n_global`` leading global tokens, the op of T5BlockAttention
     (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout.
 
     ``key_splits``: hand the library a workspace so that the global rows (which attend every key) are
-    spread over the device as key splits and merged; False keeps them in one workgroup per (batch, head)."""
+    spread over the device as key splits and merged; False keeps them in one workgroup per (batch, head).
+    ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence, masked the way the reference lays its
+    padding mask over the key list (attentions.py:722-732); the global rows see every key regardless (:788-800)."""
     return _sparse(L.PATTERN_BLOCK, q, k, v, bias, block_len, n_global, None, None, sm_scale, NUM_BUCKETS,
-                   MAX_DISTANCE, key_splits=key_splits, exact_scores=exact_scores)
+                   MAX_DISTANCE, key_splits=key_splits, exact_scores=exact_scores, seq_lens=seq_lens)
 
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
                                                 sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128, seq_lens=None,
-                                                exact_scores=None):
+                                                exact_scores=None, seq_starts=None):
     """Sliding window plus side tokens, the op of T5TransientGlobalAttention
     (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D).
-    ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence; a sequence of n tokens has
-    n // global_block_size side tokens (src/turbot5/model/utils.py:191-237) and its keys end at n."""
+    ``seq_lens`` / ``seq_starts`` (B,) int32: the tokens of sequence b are the rows [start, start + len); it has
+    (start + len) // global_block_size - start // global_block_size side tokens
+    (src/turbot5/model/utils.py:191-237 for one run of tokens) and only its own rows as keys."""
     return _sparse(L.PATTERN_TGLOBAL, q, k, v, bias, block_len, global_block_size, side_k, side_v, sm_scale,
-                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens, exact_scores=exact_scores)
+                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1,
-             residual: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None):
+             residual: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None,
+             seq_starts: Optional[torch.Tensor] = None):
     """T5 RMS norm over the last dimension (src/turbot5/model/modules.py:51-59).
 
     With ``residual`` (same shape and dtype as x, group 1) the kernel normalises ``x + residual`` and
@@ -408,8 +415,9 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     ``group`` > 1: x is (B, L, d) and row r of the (B, L // group, d) result is the norm of the sum of
     rows [r*group, (r+1)*group) of its sequence, trailing rows joining the last group: the side-token
     producer of transient-global attention (src/turbot5/model/utils.py:249-258, :206-212).
-    ``seq_lens`` (B,) int32 for x of shape (B, L, d), not together with ``residual``: valid rows of each right-padded sequence; a sequence of n rows
-    has n // group groups (rows past the last full one join it), output rows past them are zero.
+    ``seq_lens`` / ``seq_starts`` (B,) int32 for x of shape (B, L, d), not together with ``residual``: the rows
+    [start, start + len) of each sequence are its tokens (start defaults to 0); it has one group per group end among
+    them, the last group taking every token from its first row on; output rows past the groups are zero.
     The result has the weight's dtype when that is 16 bit, else fp32, as torch promotes the reference code."""
     if not (x.is_cuda and weight.is_cuda):
         raise RuntimeError("x and weight must be on a ROCm device: this path has no CPU implementation")
@@ -451,6 +459,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
                 or seq_lens.device != x.device or not seq_lens.is_contiguous():
             raise ValueError("seq_lens must be a contiguous int32 tensor of shape (B,) on the device of x, without residual")
         a.seq_lens = seq_lens.data_ptr()
+        if seq_starts is not None:
+            if seq_starts.dtype != torch.int32 or seq_starts.shape != (batches,) or seq_starts.device != x.device \
+                    or not seq_starts.is_contiguous():
+                raise ValueError("seq_starts must be a contiguous int32 tensor of shape (B,) on the device of x")
+            a.seq_starts = seq_starts.data_ptr()
+    elif seq_starts is not None:
+        raise ValueError("seq_starts needs seq_lens")
     total = None
     if r2 is not None:
         total = torch.empty(x.shape, dtype=x.dtype, device=x.device)
