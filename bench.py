@@ -24,6 +24,8 @@ inputs resident in HBM.  Prints ONE JSON line:
 
 --leg NAME runs one kernel K times and nothing else, for profiling:
     dense:BxL[c]  local  block  tglobal  splitk  varlen  varlen_causal  copy
+--leg NAME --timeline does the same with the measurement build of the library (`python -m turbot5_amd.build --trace`)
+and prints where the work items of the last launch spent their shader-clock cycles.
 """
 import argparse
 import json
@@ -52,6 +54,30 @@ def measured_traffic_bytes():
         return float(m.group(1)) if m else None
     except OSError:
         return None
+
+
+def device_max_clock_ghz():
+    """Maximum shader clock of the first GPU agent that rocminfo lists (GHz), or None."""
+    import subprocess
+    try:
+        txt = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    gpu = False
+    for line in txt.splitlines():
+        if "Device Type:" in line:
+            gpu = "GPU" in line
+        m = re.search(r"Max Clock Freq\. \(MHz\):\s*(\d+)", line)
+        if m and gpu:
+            return int(m.group(1)) / 1000.0
+    # the clock line comes before the device type line of an agent: second pass keyed on the agent's name
+    blocks = txt.split("*******")
+    for blk in blocks:
+        if "Device Type:             GPU" in blk or re.search(r"Device Type:\s+GPU", blk):
+            m = re.search(r"Max Clock Freq\. \(MHz\):\s*(\d+)", blk)
+            if m:
+                return int(m.group(1)) / 1000.0
+    return None
 
 
 def make_inputs(torch, dev, b, h, l, d, seed=0):
@@ -431,7 +457,7 @@ def cpu_baseline(torch, samples, seconds_budget=24.0):
 
 
 # ---------------------------------------------------------------------------------------------------------------
-def run_leg(torch, dev, name, steps, warmup):
+def run_leg(torch, dev, name, steps, warmup, timeline=False):
     """One kernel, K launches, for profiling runs."""
     from turbot5_amd import ops
     if name == "copy":
@@ -472,8 +498,50 @@ def run_leg(torch, dev, name, steps, warmup):
     else:
         raise SystemExit(f"unknown leg {name!r}")
     _, ms = time_kernel(torch, f, steps, warmup)
-    return {"leg": name, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
-            "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    out = {"leg": name, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
+           "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    if timeline:
+        out["timeline"] = read_timeline(torch, f)
+    return out
+
+
+def read_timeline(torch, fn):
+    """Cycle stamps of the work items of ONE launch from the measurement build (see T5A_STAMP in attn_fwd.hip)."""
+    import ctypes as C
+    import numpy as np
+    from turbot5_amd import _lib
+    lib = _lib.load()
+    items, slots = 4096, 16
+    buf = np.zeros(items * slots, dtype=np.uint64)
+    torch.cuda.synchronize()
+    lib.t5a_trace_read(buf.ctypes.data_as(C.c_void_p), 1)       # clear what earlier launches left
+    fn()
+    torch.cuda.synchronize()
+    rc = lib.t5a_trace_read(buf.ctypes.data_as(C.c_void_p), 0)
+    t = buf.reshape(items, slots).astype(np.int64)
+    t = t[t[:, 0] != 0]
+    if rc != 0 or len(t) == 0:
+        return {"error": f"no stamps (rc {rc})"}
+    names = ["entry -> first requests issued", "-> LUT barrier passed", "-> first score product (tile loop starts)"]
+    res = {"workgroups_stamped": int(len(t)), "unit": "shader-clock cycles, median over workgroups", "phases": []}
+    prev = t[:, 0]
+    for i in range(1, 12):
+        ok = t[:, i] != 0
+        if not ok.any():
+            break
+        label = names[i - 1] if i <= 3 else ("-> end of a q tile's tile loop" if i % 2 == 0 else "-> next q tile of the run set up")
+        res["phases"].append({"stamp": i, "what": label, "cycles": int(np.median((t[:, i] - prev)[ok])), "workgroups": int(ok.sum())})
+        prev = np.where(ok, t[:, i], prev)
+    fast = t[:, 14] > 0
+    if fast.any():      # wavefront 0's fast steps, split at the step's barrier
+        n = t[fast, 14].astype(float)
+        res["fast_steps"] = {"per_work_item": float(np.median(n)),
+                             "cycles_own_work_per_step": round(float(np.median(t[fast, 12] / n)), 1),
+                             "cycles_waiting_at_the_barrier_per_step": round(float(np.median(t[fast, 13] / n)), 1)}
+    total = t[:, :12].max(axis=1) - t[:, 0]
+    res["work_item_total"] = {"median": int(np.median(total)), "min": int(total.min()), "max": int(total.max())}
+    # the counters of different XCDs are not synchronised: only differences inside one workgroup mean anything
+    return res
 
 
 def main():
@@ -487,6 +555,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and its checks")
     ap.add_argument("--leg", default=None, metavar="NAME",
                     help="run only one kernel: dense:BxL[c], local, block, tglobal, splitk, varlen, varlen_causal, copy")
+    ap.add_argument("--timeline", action="store_true",
+                    help="with --leg: use the measurement build (libt5attn_trace.so) and print the work items' cycle stamps")
     ap.add_argument("--full", action="store_true", help="accepted for compatibility: the default run is the full one")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -494,6 +564,12 @@ def main():
         sys.exit(2)
 
     import torch
+    if args.timeline:
+        from turbot5_amd import _lib, build as t5a_build
+        if not args.leg or not os.path.exists(t5a_build.TRACE_LIB):
+            print("--timeline needs --leg and the measurement build: python -m turbot5_amd.build --trace", file=sys.stderr)
+            sys.exit(2)
+        _lib.LIB_PATH = t5a_build.TRACE_LIB
     from turbot5_amd.ops import flash_attention_with_fusing_bias
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
@@ -501,7 +577,7 @@ def main():
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(dev)
     if args.leg:
-        print(json.dumps(run_leg(torch, dev, args.leg, args.steps, args.warmup)))
+        print(json.dumps(run_leg(torch, dev, args.leg, args.steps, args.warmup, args.timeline)))
         return
 
     samples = []
@@ -530,7 +606,7 @@ def main():
             extra.update(model_workloads(torch, dev, args.steps))
 
     # the peak the device itself implies: compute units x 4096 dense bf16 FLOP per clock x its maximum clock
-    clock_ghz = props.clock_rate / 1e6 if getattr(props, "clock_rate", 0) else None
+    clock_ghz = props.clock_rate / 1e6 if getattr(props, "clock_rate", 0) else device_max_clock_ghz()
     device_peak = round(props.multi_processor_count * 4096 * clock_ghz / 1e3, 1) if clock_ghz else None
     line = {
         "metric": "fused-bias attn fwd TFLOP/s + % MFMA peak; T5-base encoder tokens/s @8k",

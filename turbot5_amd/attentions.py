@@ -484,6 +484,9 @@ class T5TransientGlobalAttention(_SparseBase):
 
 
 T5ATTENTION_TYPES = {
+    # 'basic' is the reference's eager T5Attention (attentions.py:36-257): the same math as 'flash', which is what
+    # runs here (no attention weights, head mask or attention dropout; those raise NotImplementedError)
+    "basic": T5FlashAttention,
     "flash": T5FlashAttention,
     "triton-basic": T5FlashAttention,   # same math as 'flash'; the materialised-bias kernel is not rebuilt
     "local": T5LocalAttention,

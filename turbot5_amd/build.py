@@ -49,19 +49,28 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
-def build(verbose: bool = False, jobs: int = 8, extra_flags=()) -> str:
-    """Compile every translation unit and link the shared library; returns its path."""
-    os.makedirs(OBJ, exist_ok=True)
+TRACE_LIB = os.path.join(HERE, "libt5attn_trace.so")
+
+
+def build(verbose: bool = False, jobs: int = 8, extra_flags=(), trace: bool = False) -> str:
+    """Compile every translation unit and link the shared library; returns its path.
+
+    ``trace``: a second library, libt5attn_trace.so, whose bf16 attention kernels stamp the shader clock at a few
+    points of every work item (``bench.py --timeline`` reads them); the shipped library carries none of that."""
+    obj_dir = os.path.join(OBJ, "trace") if trace else OBJ
+    os.makedirs(obj_dir, exist_ok=True)
     hipcc = _hipcc()
+    flags = [*FLAGS, *extra_flags] + (["-DT5A_TRACE"] if trace else [])
     cmds = []
     for obj, src, defs in UNITS:
-        cmds.append([hipcc, *FLAGS, *extra_flags, *defs, "-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ, obj)])
+        cmds.append([hipcc, *flags, *defs, "-c", os.path.join(CSRC, src), "-o", os.path.join(obj_dir, obj)])
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda c: _run(c, verbose), cmds))
-    objs = [os.path.join(OBJ, o) for o, _, _ in UNITS]
-    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB, *objs], verbose)
-    return LIB
+    objs = [os.path.join(obj_dir, o) for o, _, _ in UNITS]
+    lib = TRACE_LIB if trace else LIB
+    _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", lib, *objs], verbose)
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, trace="--trace" in sys.argv))

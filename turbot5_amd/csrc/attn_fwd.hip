@@ -54,6 +54,34 @@
 
 namespace t5a {
 
+// Timeline of a work item, for measurements only (build with -DT5A_TRACE, `python -m turbot5_amd.build --trace`): the
+// first thread of every workgroup of the bf16 kernels stamps the shader clock at a few points; t5a_trace_read copies
+// the stamps out.  Slot 0: kernel entry, 1: first key/value and query requests issued, 2: the LUT barrier passed,
+// 3: first score product formed (the tile loop starts), 4..: end of each q tile's tile loop and, for runs of q tiles,
+// the start of the next one's.  The shipped library has none of this.
+#if defined(T5A_TRACE) && T5A_UNIT_DTYPE == 0
+constexpr int kTraceSlots = 16, kTraceItems = 4096;
+__device__ unsigned long long t5a_trace_buf[kTraceItems * kTraceSlots];
+#define T5A_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < kTraceItems && (i) < kTraceSlots) \
+        t5a_trace_buf[(size_t)blockIdx.x * kTraceSlots + (i)] = __builtin_readcyclecounter(); } while (0)
+// ... and the time of the fast steps of wavefront 0, split at the step's barrier: slot 12 holds the cycles from a
+// barrier's end to the next wait (the step's own work), slot 13 the cycles in the wait for the tile requests and the
+// barrier, slot 14 the number of fast steps
+#define T5A_PHASE_VARS unsigned long long tr_last = 0, tr_acc[2] = {0, 0}; unsigned tr_steps = 0
+#define T5A_PHASE_START() do { tr_last = __builtin_readcyclecounter(); } while (0)
+#define T5A_PHASE(k) do { const unsigned long long now_ = __builtin_readcyclecounter(); tr_acc[k] += now_ - tr_last; \
+        tr_last = now_; tr_steps += (k); } while (0)
+#define T5A_PHASE_STORE() do { if (threadIdx.x == 0 && blockIdx.x < kTraceItems) { \
+        unsigned long long* s_ = t5a_trace_buf + (size_t)blockIdx.x * kTraceSlots; \
+        s_[12] = tr_acc[0]; s_[13] = tr_acc[1]; s_[14] = tr_steps; } } while (0)
+#else
+#define T5A_STAMP(i)
+#define T5A_PHASE_VARS
+#define T5A_PHASE_START()
+#define T5A_PHASE(k)
+#define T5A_PHASE_STORE()
+#endif
+
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -82,6 +110,11 @@ template <> struct Elem<__bf16> {
         }
         return acc;
     }
+    static __device__ __forceinline__ float sum4(v4 x, float acc) {
+        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[0], x[1]}, one, acc, false);
+        return __builtin_amdgcn_fdot2_f32_bf16(bf16x2{x[2], x[3]}, one, acc, false);
+    }
 };
 template <> struct Elem<_Float16> {
     using v8 = f16x8; using v4 = f16x4;
@@ -96,6 +129,11 @@ template <> struct Elem<_Float16> {
             acc = __builtin_amdgcn_fdot2(pr, one, acc, false);
         }
         return acc;
+    }
+    static __device__ __forceinline__ float sum4(v4 x, float acc) {
+        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        acc = __builtin_amdgcn_fdot2(f16x2{x[0], x[1]}, one, acc, false);
+        return __builtin_amdgcn_fdot2(f16x2{x[2], x[3]}, one, acc, false);
     }
 };
 template <> struct Elem<float> {
@@ -297,6 +335,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                  "s"(p.k_sb), "s"(p.k_sh), "s"(p.k_sr), "s"(p.v_sb), "s"(p.v_sh), "s"(p.v_sr));
     asm volatile("" :: "s"(p.o_sb), "s"(p.o_sh), "s"(p.o_sr), "s"(p.t_sbucket), "s"(p.t_shead),
                  "s"(p.bs.bidirectional), "s"(p.bs.nb), "s"(p.bs.max_exact), "s"(p.bs.n_thr), "s"(p.bs.sat));
+    T5A_STAMP(0);
+    int trace_slot = 4;
+    (void)trace_slot;
     int w = 0;
     const bool planned = MODE == kPacked && p.plan != nullptr;
     if (planned) {
@@ -481,28 +522,27 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // and a block's segment spans a whole block; tiles outside the keys that exist read as zeros and are skipped
     // or masked.
     int seg_nt[2] = {0, 0};
-    int hole_lo = 0, hole_span = 0;   // block pattern, padded sequence: own-block keys [hole_lo, hole_lo + hole_span) are masked
+    // block pattern, right-padded sequence: the own-block keys [lo, lo + span) that the rows of block blk do not see.
+    // The reference lays its additive padding mask out as [own block | global tokens] over keys that are laid out
+    // [global tokens | own block] (src/turbot5/model/attentions.py:722-732 against :807-814): list column
+    // c < block_len is masked iff token blk * block_len + c is padding, the last G columns never are (except in
+    // block 0, where they always are).  valid = how many of the first block_len list columns stay.  (Derived from
+    // n_valid where a tile is classified or masked, rather than kept: the pattern's tile loop has no registers left.)
+    auto block_valid = [&]() { return max(0, min(p.block_len, n_valid - blk * p.block_len)); };
+    auto block_hole = [&](int& lo, int& span) {
+        const int head = max(block_valid() - p.aux, 0);   // own-block keys before the masked range
+        lo = blk * p.block_len + head;
+        span = blk == 0 ? 0 : max(0, p.block_len - p.aux - head);
+    };
     auto set_qtile = [&](int q_tile) {
         if (MODE == kBlock && !gsplit) {
             blk = q_tile / tpb;
             i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
             row_end = min(Mseq, (blk + 1) * p.block_len);
             seg_start[1] = blk * p.block_len;
-            // The reference lays its additive padding mask out as [own block | global tokens] over keys that are
-            // laid out [global tokens | own block] (src/turbot5/model/attentions.py:722-732 against :807-814): list
-            // column c < block_len is masked iff token blk * block_len + c is padding, the last G columns never are
-            // (except in block 0, where they always are).  valid = how many of the first block_len list columns stay.
-            const int valid = max(0, min(p.block_len, n_valid - blk * p.block_len));
+            const int valid = block_valid();
             seg_end[0] = min(p.aux, valid);
-            const int head = max(valid - p.aux, 0);           // own-block keys before the masked range
-            if (blk == 0) {
-                seg_end[1] = min(p.block_len - p.aux, head);
-                hole_span = 0;
-            } else {
-                seg_end[1] = (blk + 1) * p.block_len;
-                hole_lo = blk * p.block_len + head;
-                hole_span = max(0, p.block_len - p.aux - head);
-            }
+            seg_end[1] = blk == 0 ? min(p.block_len - p.aux, max(valid - p.aux, 0)) : (blk + 1) * p.block_len;
         } else {
             i0 = q_tile * BM;
             row_end = Mseq;
@@ -760,6 +800,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     } else if (has_bias && col_in_lanes && lane < nbt && !lut_cached) {
         tcol = load_table(p.table, p.table_dtype, (int64_t)lane * p.t_sbucket + (int64_t)h * p.t_shead) * log2e;
     }
+    T5A_STAMP(1);
     // request the first tiles: they arrive while the bias LUT is built
     if constexpr (DMA) {
         if constexpr (QDMA) {
@@ -794,6 +835,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         for (int idx = tid; idx < NSV * V_TILE; idx += NTHREADS) Vs[idx] = (T)0.0f;
     }
     __syncthreads();
+    T5A_STAMP(2);
     const float c_neg = has_bias ? lut[0] : 0.f;                 // every key far before the query
     const float c_pos = has_bias ? lut[qlen - 1] : 0.f;          // every key far after it (non-causal)
 
@@ -972,8 +1014,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             c.need_mask = c.need_mask || c.j0 < key_lo;
         }
         if (win && !win_lut) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
-        if (MODE == kBlock && c.sg == 1 && hole_span > 0)
+        if (MODE == kBlock && c.sg == 1 && n_valid < Nseq) {
+            int hole_lo, hole_span;
+            block_hole(hole_lo, hole_span);
             c.need_mask = c.need_mask || (c.j0 < hole_lo + hole_span && c.j0 + BN > hole_lo);
+        }
         c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
         if constexpr (win_lut) c.side = 0;
         return c;
@@ -1063,9 +1108,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
 
     // S^T = K Q^T + C for one tile, C = bias - running max (cm must be current for constant tiles)
-    auto compute_s = [&](const TileClass& c, int buf, const v8 (&ka)[NT][KS], f32x16 (&st)[NT]) {
+    auto lut_acc = [&](const TileClass& c, f32x16 (&st)[NT]) {
         const int qpos = lane_qpos(c.sg);
-        if (c.use_lut) {
+        {
             const float m_neg = -m_run * inv_c1;
             const int e0 = c.j0 + 4 * hh - qpos + padl;
             const float* lb = lut + (e0 & 3) * qlen;
@@ -1092,6 +1137,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     }
             }
         }
+    };
+    auto compute_s = [&](const TileClass& c, int buf, const v8 (&ka)[NT][KS], f32x16 (&st)[NT]) {
+        if (c.use_lut) lut_acc(c, st);
         if constexpr (F32) {
             const T* ks = Ks + buf * K_TILE;
             if (!c.use_lut) {
@@ -1128,7 +1176,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
 
     // mask, row max, lazy raise of the running max; returns true when m_run changed
-    auto softmax_head = [&](const TileClass& c, f32x16 (&st)[NT]) {
+    // mask of a tile that needs one (the first part of the softmax head)
+    auto head_mask = [&](const TileClass& c, f32x16 (&st)[NT]) {
         if (c.need_mask) {   // keys past the end of the segment, or outside the window
             const int s_end = (c.sg ? seg_end[1] : seg_end[0]);
             const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0 && !win_lut;
@@ -1140,7 +1189,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const unsigned span = (unsigned)max(hi - lo, 0);
             const int jl = c.j0 + 4 * hh - lo;
             // block pattern on a padded sequence: a range of the own block's keys that the rows do not see
-            const unsigned hspan = (MODE == kBlock && c.sg == 1) ? (unsigned)hole_span : 0u;
+            int hole_lo = 0, hole_span = 0;
+            if (MODE == kBlock && c.sg == 1) block_hole(hole_lo, hole_span);
+            const unsigned hspan = (unsigned)hole_span;
             const int jh = c.j0 + 4 * hh - hole_lo;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
@@ -1152,6 +1203,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     st[nt][r] = keep ? st[nt][r] : -INFINITY;
                 }
         }
+    };
+    // the two parts of the head after the mask: the maximum of this lane's half of the row's keys (the other half
+    // sits in lane ^ 32 and is only consulted in the rare block: "some lane of the wavefront must raise" is the
+    // same question for halves and for rows) ...
+    auto head_max = [&](const f32x16 (&st)[NT]) {
         // st already holds (score - m_run)
         float pm[4];   // four independent partial maxima: short dependency chains
 #pragma unroll
@@ -1162,10 +1218,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int x = 0; x < 4; ++x) pm[c] = max_ieee(pm[c], st[nt][4 * c + x]);
-        // this lane's half of the row's keys; the other half sits in lane ^ 32 and is only consulted in the
-        // rare block: "some lane of the wavefront must raise" is the same question for halves and for rows
-        const float mh = max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3]));
-        if (__any((mh > raise_limit<T>()) || (!started && mh > -INFINITY))) {
+        return max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3]));
+    };
+    // ... and the lazy raise of the running max, when some lane asks for it; returns true when m_run changed.  (The
+    // last step of a run of fast steps forms a product past the last tile: it calls this with trigger == false,
+    // which leaves the running state alone.)
+    auto head_trigger = [&](float mh) { return __any((mh > raise_limit<T>()) || (!started && mh > -INFINITY)) != 0; };
+    auto head_raise = [&](f32x16 (&st)[NT], float mh, bool trigger) {
+        if (trigger) {
             asm volatile("");   // keep this rare block a real branch
             const float mx = xhalf_max(mh);
             // a row's first finite scores: the running max stays at 0 when they are moderate (probabilities
@@ -1193,6 +1253,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
         return false;
     };
+    auto softmax_head = [&](const TileClass& c, f32x16 (&st)[NT]) {
+        head_mask(c, st);
+        const float mh = head_max(st);
+        return head_raise(st, mh, head_trigger(mh));
+    };
 
     // P = exp2(S^T);  O^T += V^T P^T
     // per-lane part of the transposing V reads (LDS-DMA path): within a group of 16 lanes, lane
@@ -1211,7 +1276,40 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     auto compute_pv = [&](int buf, f32x16 (&st)[NT]) {
         const T* vs = Vs + buf * V_TILE;
-        if constexpr (DMA) {
+        if constexpr (DMA && D == 64) {
+            // Four groups of 16 keys.  The V^T fragments of group g + 1 are requested before the exponentials of
+            // group g, into a second set of registers, so that no product waits for the LDS; the scheduling fences
+            // keep the requests where they are (left alone, the compiler puts each one directly before its
+            // product when registers are scarce, and every product then waits a full LDS round trip).
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            auto vread = [&](int g, int dt) {
+                const T* a0 = vs + vtr_off[dt] + 16 * g * D;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
+                return __builtin_bit_cast(v8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            };
+            v8 vf[2][DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vf[0][dt] = vread(0, dt);
+#pragma unroll
+            for (int g = 0; g < 2 * NT; ++g) {
+                const int nt = g >> 1, u = g & 1;
+                if (g + 1 < 2 * NT) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) vf[(g + 1) & 1][dt] = vread(g + 1, dt);
+                }
+                __builtin_amdgcn_sched_barrier(0x40F);   // ALU and matrix instructions may cross, LDS reads may not
+                f32x8 pv;
+#pragma unroll
+                for (int x = 0; x < 8; ++x) pv[x] = __builtin_amdgcn_exp2f(st[nt][8 * u + x]);
+                const v8 pb = __builtin_convertvector(pv, v8);
+                if (u == 0) l_run = E::sum8(pb, l_run); else l_alt = E::sum8(pb, l_alt);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) ot[dt] = E::mfma(vf[g & 1][dt], pb, ot[dt]);
+                __builtin_amdgcn_sched_barrier(0x40F);
+            }
+        } else if constexpr (DMA) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -1274,10 +1372,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
 
     // ---------------------------------------------------------------- software pipeline
-    // Step t:   softmax head of tile t  ->  S MFMAs of tile t+1  ->  exp / PV MFMAs of tile t.
-    // The S product of the next tile is independent of the exp work of the current one, so the
-    // matrix pipe and the vector ALUs overlap inside one wavefront.  K tiles are staged two steps
-    // ahead and V tiles one step ahead, each in two LDS buffers, with one barrier per step.
+    // Step t:   S MFMAs of tile t+1 with the exponentials of tile t  ->  PV MFMAs of tile t with the softmax head
+    // (row maxima, row sums) of tile t+1.
+    // A wavefront issues in order and the matrix pipe takes one 32x32x16 product per 32 cycles, so a burst of
+    // products stalls its wavefront while the vector ALUs idle, and a stretch of vector work leaves the matrix pipe
+    // idle: each half of the step pairs matrix work with vector work that does not depend on it, interleaved
+    // instruction by instruction (the fast steps fix that order with scheduling groups).  K tiles are staged two
+    // steps ahead and V tiles one step ahead, each in two LDS buffers, with one barrier per step.
     //
     // LDS-DMA path: K(t+4) and V(t+3) are requested in step t into four-stage rings; every step
     // issues the same number of loads per wavefront (2 * SPW; tiles past the end fetch zeros), so
@@ -1300,10 +1401,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         __syncthreads();
     }
     if (tc.side != 0) refill_cm(tc.side);
+    T5A_PHASE_VARS;
+    bool head_refill = false;   // the head of the current tile moved the running max: cm is stale
     if (ntiles > 0 && !tc.skip) {
         v8 ka0[NT][KS];
         read_k(0, ka0);
         compute_s(tc, 0, ka0, sta);
+        head_refill = softmax_head(tc, sta);
     }
     if constexpr (QDMA) wait_vmcnt<3 * G::SPW>();   // K1 has landed; V1 K2 V2 may still be in flight
     __syncthreads();   // the first step overwrites the K buffer this product was read from
@@ -1322,11 +1426,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const TileClass nx = classify(t + 1);
         v8 ka[NT][KS];
         if (!nx.skip) read_k(kbuf_next, ka);
-        bool refill = false;
-        if (!tc.skip) refill = softmax_head(tc, st);
-        if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        head_refill = false;
         if (!nx.skip) compute_s(nx, kbuf_next, ka, st_next);
         if (!tc.skip) compute_pv(vbuf, st);
+        if (!nx.skip) head_refill = softmax_head(nx, st_next);
         tc = nx;
         if constexpr (DMA) {
             wait_vmcnt<4 * G::SPW>();   // everything but the last two steps' requests
@@ -1335,6 +1439,66 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             if (t + 2 < ntiles) store_tile_k(t & 1);
             if (t + 1 < ntiles) store_tile_v((t + 1) & 1);
             __syncthreads();
+        }
+    };
+    // Both halves of a fast step at head_dim 64 as one instruction stream: sixteen groups, each one matrix product
+    // with the vector work that runs beside it, kept in this order by scheduling fences (what the compiler does with
+    // the same statements unfenced: all exponentials first, all maxima last, and the matrix pipe idle meanwhile).
+    // The first two S products (k-step 0 of both key blocks) are issued by the caller, which knows their accumulator
+    // input.
+    auto fused_halves = [&](bool live, int vstage, const v8 (&ka)[NT][KS], f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        if constexpr (DMA && D == 64) {
+            static_assert(NT == 2 && KS == 4 && DT == 2, "four groups of 16 keys, two products each");
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const T* vs = Vs + vstage * V_TILE;
+            v4 ph[8];        // P, four keys per entry
+            v8 vf[4][DT];    // V^T fragments
+            auto vread = [&](int g, int dt) {
+                const T* a0 = vs + vtr_off[dt] + 16 * g * D;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
+                vf[g][dt] = __builtin_bit_cast(v8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            // first half: exponentials of tile t beside the S products of tile t+1; the V^T fragments of the first
+            // 32 keys go into the registers of K fragments that are done with
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                f32x4 pv;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) pv[x] = __builtin_amdgcn_exp2f(st[i >> 2][4 * (i & 3) + x]);
+                ph[i] = __builtin_convertvector(pv, v4);
+                if (i >= 2) st_next[i & 1] = E::mfma(ka[i & 1][i >> 1], qf[i >> 1], st_next[i & 1]);
+                if (i >= 4) vread((i - 4) >> 1, (i - 4) & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (exact) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) st_next[nt][r] *= p.c1;
+            }
+            // second half: PV products of tile t beside its row sums and the row maxima of tile t+1
+            float pm[4];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int g = i >> 1, dt = i & 1;
+                const v8 pb = __builtin_shufflevector(ph[2 * g], ph[2 * g + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                ot[dt] = E::mfma(vf[g][dt], pb, ot[dt]);
+                if (i < 4) vread(2 + (i >> 1), i & 1);
+                if ((g & 1) == 0) l_run = E::sum4(ph[i], l_run); else l_alt = E::sum4(ph[i], l_alt);
+                // maxima: chain c takes the slots 4c .. 4c+3 of both key blocks, two of them per group
+                {
+                    const int nt = i >> 2, c = i & 3;
+                    const float a = max_ieee(st_next[nt][4 * c], st_next[nt][4 * c + 1]);
+                    const float b2 = max_ieee(st_next[nt][4 * c + 2], st_next[nt][4 * c + 3]);
+                    pm[c] = nt == 0 ? max_ieee(a, b2) : max_ieee(pm[c], max_ieee(a, b2));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const float mh = max_ieee(max_ieee(pm[0], pm[1]), max_ieee(pm[2], pm[3]));
+            head_refill = head_raise(st_next, mh, live & head_trigger(mh));
         }
     };
     // Fast step (LDS-DMA path): tiles t and t+1 are neither skipped nor masked, so the step is the
@@ -1346,17 +1510,32 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
-        TileClass cur;
-        cur.sg = tc.sg; cur.j0 = tc.j0; cur.side = 0; cur.skip = false; cur.use_lut = false; cur.need_mask = false;
         const TileClass nx = classify(t + 1);
-        const bool refill = softmax_head(cur, st);
-        if (refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
-        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): one wait for all K fragments instead of one per MFMA
-        compute_s(nx, (ST + 1) & 3, ka, st_next);
-        compute_pv(ST, st);
+        if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        head_refill = false;
+        const bool live = !nx.skip;   // false in the last step of a run that ends with the last tile
+        if constexpr (D == 64) {
+            if (nx.use_lut) {
+                lut_acc(nx, st_next);
+                st_next[0] = E::mfma(ka[0][0], qf[0], st_next[0]);
+                st_next[1] = E::mfma(ka[1][0], qf[0], st_next[1]);
+            } else {
+                st_next[0] = E::mfma(ka[0][0], qf[0], cm);   // cm stays live: untied accumulator input
+                st_next[1] = E::mfma(ka[1][0], qf[0], cm);
+            }
+            fused_halves(live, ST, ka, st, st_next);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): one wait for all K fragments instead of one per MFMA
+            compute_s(nx, (ST + 1) & 3, ka, st_next);
+            compute_pv(ST, st);
+            const float mh = head_max(st_next);
+            head_refill = head_raise(st_next, mh, live & head_trigger(mh));
+        }
         tc = nx;
+        T5A_PHASE(0);
         wait_vmcnt<4 * G::SPW>();
         barrier_lds_only();
+        T5A_PHASE(1);
     };
     // number of consecutive tiles from t on that are neither skipped nor masked
     auto plain_run = [&](int t) {
@@ -1421,6 +1600,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
     };
 
+    T5A_STAMP(3);
     if constexpr (RUNS) prefetch_q(qt + 1);
     bool interior = first_interior;   // the current q tile's classes hold for any q tile away from the ends of the sequence
     for (;;) {
@@ -1437,6 +1617,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     tc = classify(t);
                     if constexpr (DENSE) cursor_seek(t + 4, t + 3);
                 }
+                if (quads > 0) T5A_PHASE_START();
                 while (quads > 0) {
                     fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
                     fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
@@ -1450,6 +1631,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             if (t + 1 < ntiles) step(t + 1, stb, sta);
             t += 2;
         }
+        T5A_STAMP(trace_slot); ++trace_slot;
+        T5A_PHASE_STORE();
         if constexpr (!RUNS) {
             store_rows();
             break;
@@ -1487,12 +1670,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             if (!(interior && was_interior)) fill_classes();
             tc = classify(0);
             if (tc.side != 0) refill_cm(tc.side);
+            head_refill = false;
             if (!tc.skip) {
                 v8 ka0[NT][KS];
                 read_k(tbase % NSK, ka0);
                 compute_s(tc, tbase % NSK, ka0, sta);
+                head_refill = softmax_head(tc, sta);
             }
             barrier_lds_only();   // the first step's request overwrites the K stage this product was read from
+            T5A_STAMP(trace_slot); ++trace_slot;
         }
     }
     if constexpr (!RUNS) {
@@ -1596,3 +1782,16 @@ hipError_t launch_fwd_f16(const FwdParams& p, int D, int mode, bool causal, hipS
 #endif
 
 }  // namespace t5a
+
+#if defined(T5A_TRACE) && T5A_UNIT_DTYPE == 0
+// measurement builds only: copies the stamps (kTraceItems x kTraceSlots 64-bit shader-clock values) to the host
+extern "C" int t5a_trace_read(unsigned long long* out, int clear) {
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(t5a::t5a_trace_buf), sizeof(unsigned long long) * t5a::kTraceItems * t5a::kTraceSlots);
+    if (e == hipSuccess && clear) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(t5a::t5a_trace_buf));
+        if (e == hipSuccess) e = hipMemset(ptr, 0, sizeof(unsigned long long) * t5a::kTraceItems * t5a::kTraceSlots);
+    }
+    return (int)e;
+}
+#endif
