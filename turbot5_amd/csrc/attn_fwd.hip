@@ -638,6 +638,44 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             }
         }
     };
+    // Runs of q tiles (one segment): the K and the V requests each walk the tiles of the run in order, so each keeps
+    // a cursor -- first key, tile index inside its q tile, q tile -- that a request advances with a few scalar
+    // instructions (where tile_of divides).  A request past the run's last q tile fills its stage with zeros.
+    int rq_j0[2] = {0, 0}, rq_ts[2] = {0, 0}, rq_q[2] = {0, 0}, rq_stage[2] = {0, 0};   // [0]: K, [1]: V
+    int rq_koff[G::SPW], rq_voff[G::SPW];   // this lane's byte offsets inside a tile
+#pragma unroll
+    for (int c = 0; c < G::SPW; ++c) rq_koff[c] = rq_voff[c] = 0;
+    if constexpr (RUNS) {
+#pragma unroll
+        for (int c = 0; c < G::SPW; ++c) {
+            const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
+            rq_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16;
+            rq_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16;
+        }
+        rq_j0[0] = rq_j0[1] = qt * BM - p.block_len + 1;
+        rq_q[0] = rq_q[1] = qt;
+    }
+    auto dma_next = [&](bool is_v, int stage = -1) {
+        if constexpr (RUNS) {
+            const int w = is_v ? 1 : 0;
+            const int j0 = w ? rq_j0[1] : rq_j0[0];
+            const int q_tile = w ? rq_q[1] : rq_q[0];
+            u32x4 rs = is_v ? seg_vrw[0] : seg_krw[0];
+            if (q_tile >= qt_last) rs[2] = 0u;
+            if (stage < 0) stage = w ? rq_stage[1] : rq_stage[0];
+            const unsigned base = lds_base + (is_v ? (unsigned)(stage * V_TILE) : (unsigned)(NSV * V_TILE + stage * K_TILE)) * ES;
+            const int tile_off = j0 * (is_v ? seg_vsr[0] : seg_ksr[0]);
+#pragma unroll
+            for (int c = 0; c < G::SPW; ++c)
+                lds_dma_16(rs, base + (wave * G::SPW + c) * 1024, tile_off + (is_v ? rq_voff[c] : rq_koff[c]));
+            // advance (explicit selects: an indexed private array would live in scratch memory)
+            int ts = (w ? rq_ts[1] : rq_ts[0]) + 1, nj0 = j0 + BN, nq = q_tile;
+            if (ts == ntiles) { ts = 0; nq = q_tile + 1; nj0 += BM - ntiles * BN; }
+            const int nst = ((w ? rq_stage[1] : rq_stage[0]) + 1) % (w ? NSV : NSK);
+            if (w) { rq_ts[1] = ts; rq_j0[1] = nj0; rq_q[1] = nq; rq_stage[1] = nst; }
+            else { rq_ts[0] = ts; rq_j0[0] = nj0; rq_q[0] = nq; rq_stage[0] = nst; }
+        }
+    };
     // Dense mode, fast steps: a running descriptor per tensor.  The tile's byte offset lives in the
     // descriptor (base up, readable size down, clamped at zero so that tiles past the end still read
     // zeros), advanced with a few scalar instructions per step, and the per-lane offsets are loop
@@ -773,6 +811,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                                       : (unsigned)(3 * V_TILE) * ES + (wave - 2) * 4096u;
     if constexpr (QDMA) {
         if constexpr (DENSE) { cursor_seek(0, 0); cursor_dma(0, 0); }
+        else if constexpr (RUNS) { dma_next(false); dma_next(true); }
         else { dma_tile(0, false); dma_tile(0, true); }
         const int q_row_bytes = (int)p.q_sr * ES;
         const u32x4 rs = make_rsrc_words(qp, row_end > 0 ? (unsigned)(row_end - 1) * (unsigned)q_row_bytes + D * ES : 0u);
@@ -805,11 +844,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (DMA) {
         if constexpr (QDMA) {
             if constexpr (DENSE) { cursor_dma(1, 1); cursor_dma(2, 2); }   // K1 V1, K2 V2
+            else if constexpr (RUNS) { dma_next(false); dma_next(true); dma_next(false); dma_next(true); }
             else { dma_tile(1, false); dma_tile(1, true); dma_tile(2, false); dma_tile(2, true); }
         } else if constexpr (DENSE) {
             cursor_seek(0, 0);
             cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
             dma_tile(3, false);                                     // K3
+        } else if constexpr (RUNS) {
+            for (int i = 0; i < 4; ++i) dma_next(false);
+            for (int i = 0; i < 3; ++i) dma_next(true);
         } else {
             for (int i = 0; i < 4; ++i) dma_tile(i, false);
             for (int i = 0; i < 3; ++i) dma_tile(i, true);
@@ -1411,12 +1454,17 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     if constexpr (QDMA) wait_vmcnt<3 * G::SPW>();   // K1 has landed; V1 K2 V2 may still be in flight
     __syncthreads();   // the first step overwrites the K buffer this product was read from
-    if constexpr (QDMA) dma_tile(3, false);         // K3, into the stage that held the Q rows of two wavefronts
+    if constexpr (QDMA) {   // K3, into the stage that held the Q rows of two wavefronts
+        if constexpr (RUNS) dma_next(false); else dma_tile(3, false);
+    }
 
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         const int kbuf_next = DMA ? (tbase + t + 1) % NSK : (t + 1) & 1;
         const int vbuf = DMA ? (tbase + t) % NSV : t & 1;
-        if constexpr (DMA) {
+        if constexpr (RUNS) {
+            dma_next(false);
+            dma_next(true);
+        } else if constexpr (DMA) {
             dma_tile(t + 4, false);
             dma_tile(t + 3, true);
         } else {
@@ -1426,7 +1474,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const TileClass nx = classify(t + 1);
         v8 ka[NT][KS];
         if (!nx.skip) read_k(kbuf_next, ka);
-        if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        if constexpr (!win_lut) {   // (with the window in the LUT no tile has a constant accumulator input)
+            if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        }
         head_refill = false;
         if (!nx.skip) compute_s(nx, kbuf_next, ka, st_next);
         if (!tc.skip) compute_pv(vbuf, st);
@@ -1507,11 +1557,18 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
         if constexpr (DENSE) cursor_dma(ST, (ST + 3) & 3);
+        else if constexpr (RUNS) { dma_next(false, ST); dma_next(true, (ST + 3) & 3); }
         else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
-        const TileClass nx = classify(t + 1);
-        if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        TileClass nx;
+        if constexpr (win_lut) {   // one segment, every tile takes its accumulator input from the LUT: nothing to look up
+            nx.sg = 0; nx.j0 = i0 - p.block_len + 1 + (t + 1) * BN; nx.side = 0;
+            nx.skip = t + 1 >= ntiles; nx.use_lut = true; nx.need_mask = false;
+        } else {
+            nx = classify(t + 1);
+            if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
+        }
         head_refill = false;
         const bool live = !nx.skip;   // false in the last step of a run that ends with the last tile
         if constexpr (D == 64) {
