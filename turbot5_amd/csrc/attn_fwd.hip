@@ -224,6 +224,13 @@ __device__ __forceinline__ void lds_dma_16x2(unsigned lo, unsigned hi, unsigned 
                  :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory", "m0");
 }
 
+// ... with the descriptor as it is (four scalar registers that the caller keeps)
+__device__ __forceinline__ void lds_dma_16x2(u32x4 rsrc, unsigned lds_addr, int voff0, int voff1) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
+                 "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff0), "v"(voff1), "s"(rsrc) : "memory", "m0");
+}
+
 // s_waitcnt vmcnt(N) alone (six-bit count: bits 3:0 and 15:14), the other counters left open
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -582,7 +589,6 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     int tbase = 0;                               // tiles of the run's earlier q tiles (the ring stages count on)
     __amdgpu_buffer_rsrc_t seg_krs[2], seg_vrs[2];
     u32x4 seg_krw[2], seg_vrw[2];
-    int seg_kbytes0 = 0, seg_vbytes0 = 0;   // readable bytes of segment 0
 #pragma unroll
     for (int sg = 0; sg < 2; ++sg) {
         // rows at or past this read as zero.  RUNS: one descriptor per tensor for the whole run -- all the keys of
@@ -594,7 +600,6 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         seg_vrs[sg] = make_rsrc(seg_v[sg], vb);
         seg_krw[sg] = make_rsrc_words(seg_k[sg], kb);
         seg_vrw[sg] = make_rsrc_words(seg_v[sg], vb);
-        if (sg == 0) { seg_kbytes0 = (int)kb; seg_vbytes0 = (int)vb; }
     }
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -676,50 +681,43 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             else { rq_ts[0] = ts; rq_j0[0] = nj0; rq_q[0] = nq; rq_stage[0] = nst; }
         }
     };
-    // Dense mode, fast steps: a running descriptor per tensor.  The tile's byte offset lives in the
-    // descriptor (base up, readable size down, clamped at zero so that tiles past the end still read
-    // zeros), advanced with a few scalar instructions per step, and the per-lane offsets are loop
-    // invariant.  Slices stay below 2 GiB (checked on the host), so signed 32-bit sizes do.
-    unsigned long long kcur = 0, vcur = 0;
-    int kleft = 0, vleft = 0;
+    // Dense mode: the K and V requests walk the tiles in order with per-lane running byte offsets (one vector add
+    // per request and step, where a descriptor moved along by scalar code costs the wavefront some twenty scalar
+    // instructions: a wavefront issues one instruction of any kind every four to five cycles, so scalar bookkeeping
+    // is as expensive as vector work).  The descriptors span all rows of the (batch, head): tiles past the end are
+    // out of range and arrive as zeros.  Slices stay below 2 GiB (checked on the host), so 32-bit offsets do.
     const int kstep = BN * seg_ksr[0], vstep = BN * seg_vsr[0];
     int cur_koff[G::SPW], cur_voff[G::SPW];
 #pragma unroll
     for (int c = 0; c < G::SPW; ++c) cur_koff[c] = cur_voff[c] = 0;
-    if constexpr (DMA && DENSE) {
-#pragma unroll
-        for (int c = 0; c < G::SPW; ++c) {
-            const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
-            // requests go out in pairs; the second of a pair carries an instruction offset of 1024
-            cur_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16 - (c & 1) * 1024;
-            cur_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16 - (c & 1) * 1024;
-        }
-    }
     auto cursor_seek = [&](int tk, int tv) {   // next requests: K tile tk, V tile tv
-        kcur = reinterpret_cast<unsigned long long>(seg_k[0]) + (unsigned long long)((unsigned)tk * (unsigned)kstep);
-        vcur = reinterpret_cast<unsigned long long>(seg_v[0]) + (unsigned long long)((unsigned)tv * (unsigned)vstep);
-        kleft = seg_kbytes0 - tk * kstep;
-        vleft = seg_vbytes0 - tv * vstep;
+        if constexpr (DMA && DENSE) {
+#pragma unroll
+            for (int c = 0; c < G::SPW; ++c) {
+                const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
+                // requests go out in pairs; the second of a pair carries an instruction offset of 1024
+                cur_koff[c] = r * seg_ksr[0] + (pc ^ G::kswz(r)) * 16 - (c & 1) * 1024 + tk * kstep;
+                cur_voff[c] = r * seg_vsr[0] + (pc ^ G::vrow_swz(r)) * 16 - (c & 1) * 1024 + tv * vstep;
+            }
+        }
     };
     auto cursor_dma = [&](int kstage, int vstage) {
         if constexpr (DMA) {
             const unsigned wbase = lds_base + (unsigned)wave * (1024u * G::SPW);
             if constexpr (G::SPW == 1) {   // one request per tensor and wavefront
-                const u32x4 kr = {(unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0), 0x00020000u};
-                const u32x4 vr = {(unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0), 0x00020000u};
-                lds_dma_16(kr, wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES, cur_koff[0]);
-                lds_dma_16(vr, wbase + (unsigned)(vstage * V_TILE) * ES, cur_voff[0]);
+                lds_dma_16(seg_krw[0], wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES, cur_koff[0]);
+                lds_dma_16(seg_vrw[0], wbase + (unsigned)(vstage * V_TILE) * ES, cur_voff[0]);
             } else {
 #pragma unroll
                 for (int c = 0; c + 1 < G::SPW; c += 2) {
-                    lds_dma_16x2((unsigned)kcur, (unsigned)(kcur >> 32) & 0xffffu, (unsigned)max(kleft, 0),
-                                 wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES + c * 1024u, cur_koff[c], cur_koff[c + 1]);
-                    lds_dma_16x2((unsigned)vcur, (unsigned)(vcur >> 32) & 0xffffu, (unsigned)max(vleft, 0),
-                                 wbase + (unsigned)(vstage * V_TILE) * ES + c * 1024u, cur_voff[c], cur_voff[c + 1]);
+                    lds_dma_16x2(seg_krw[0], wbase + (unsigned)(NSV * V_TILE + kstage * K_TILE) * ES + c * 1024u,
+                                 cur_koff[c], cur_koff[c + 1]);
+                    lds_dma_16x2(seg_vrw[0], wbase + (unsigned)(vstage * V_TILE) * ES + c * 1024u,
+                                 cur_voff[c], cur_voff[c + 1]);
                 }
             }
-            kcur += (unsigned)kstep; vcur += (unsigned)vstep;
-            kleft -= kstep; vleft -= vstep;
+#pragma unroll
+            for (int c = 0; c < G::SPW; ++c) { cur_koff[c] += kstep; cur_voff[c] += vstep; }
         }
     };
     // ---------------------------------------------------------------- Q fragments: loads first
@@ -1266,7 +1264,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // ... and the lazy raise of the running max, when some lane asks for it; returns true when m_run changed.  (The
     // last step of a run of fast steps forms a product past the last tile: it calls this with trigger == false,
     // which leaves the running state alone.)
-    auto head_trigger = [&](float mh) { return __any((mh > raise_limit<T>()) || (!started && mh > -INFINITY)) != 0; };
+    auto head_trigger = [&](float mh) {   // (no short-circuit: both tests are one compare, a branch around one costs more)
+        const bool hot = mh > raise_limit<T>();
+        const bool first = (!started) & (mh > -INFINITY);
+        return __any(hot | first) != 0;
+    };
     auto head_raise = [&](f32x16 (&st)[NT], float mh, bool trigger) {
         if (trigger) {
             asm volatile("");   // keep this rare block a real branch
@@ -1554,6 +1556,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // Fast step (LDS-DMA path): tiles t and t+1 are neither skipped nor masked, so the step is the
     // general one minus those cases.  ST is the step index modulo 4, which fixes every LDS stage at
     // compile time.
+    int fc_until = 0, fc_side = 0;   // dense fast steps: class of the next tile, valid for tiles below fc_until
+    bool fc_lut = false;
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
         if constexpr (DENSE) cursor_dma(ST, (ST + 3) & 3);
@@ -1565,6 +1569,16 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if constexpr (win_lut) {   // one segment, every tile takes its accumulator input from the LUT: nothing to look up
             nx.sg = 0; nx.j0 = i0 - p.block_len + 1 + (t + 1) * BN; nx.side = 0;
             nx.skip = t + 1 >= ntiles; nx.use_lut = true; nx.need_mask = false;
+        } else if constexpr (DENSE) {
+            // the class only changes at a few tile indices: look it up there, carry it along otherwise
+            if (t + 1 >= fc_until) {
+                const TileClass c = classify(t + 1);
+                fc_lut = c.use_lut; fc_side = c.side;
+                fc_until = t + 1 < d_tl ? d_tl : (t + 1 < d_tr ? d_tr : 0x7fffffff);
+            }
+            nx.sg = 0; nx.j0 = (t + 1) * BN; nx.side = fc_side;
+            nx.skip = t + 1 >= ntiles; nx.use_lut = fc_lut; nx.need_mask = false;
+            if (head_refill || (fc_side != 0 && fc_side != side_cur)) refill_cm(fc_side);
         } else {
             nx = classify(t + 1);
             if (head_refill || (nx.side != 0 && nx.side != side_cur)) refill_cm(nx.side);
@@ -1672,7 +1686,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 int quads = (t + run >= ntiles ? run : run - 1) >> 2;
                 if (quads > 0) {
                     tc = classify(t);
-                    if constexpr (DENSE) cursor_seek(t + 4, t + 3);
+                    if constexpr (DENSE) { cursor_seek(t + 4, t + 3); fc_until = 0; }
                 }
                 if (quads > 0) T5A_PHASE_START();
                 while (quads > 0) {
