@@ -364,14 +364,17 @@ static int device_compute_units() {
 // pattern is only a few steps long, about as long as the set-up of a work item, which a run pays once; longer runs
 // mean fewer workgroups.  Two workgroups fit a compute unit: count the rounds the device needs for the runs and
 // charge every round its q tiles plus one set-up.
-static void choose_runs(FwdParams* p, int mode, int dtype, int D) {
+static void choose_runs(FwdParams* p, int mode, int dtype, int D, int64_t other_items = 0) {
     p->run_len = 1;
     p->runs_per_seq = p->tiles_per_seq;
     const int64_t entries = (int64_t)p->tiles_per_seq * p->H * p->B;   // the (batch, head, q tile) list
-    const bool runs_ok = mode == kLocal && dtype != T5A_F32 && (D == 64 || D == 128);   // the geometries staged by LDS-DMA
+    // the geometries staged by LDS-DMA
+    const bool runs_ok = (mode == kLocal || mode == kBlock) && dtype != T5A_F32 && (D == 64 || D == 128);
     if (runs_ok) {
-        // as many workgroups as the device holds at once (two per compute unit), each with its share of the list
-        const int64_t slots = 2 * (int64_t)device_compute_units();
+        // as many workgroups as the device holds at once (two per compute unit), each with its share of the list;
+        // other_items: workgroups of the same launch that are not runs (the block pattern's key splits)
+        int64_t slots = 2 * (int64_t)device_compute_units() - other_items;
+        if (slots < 64) slots = 64;
         int64_t rl = (entries + slots - 1) / slots;
         if (rl > 16) rl = 16;
         if (rl < 1) rl = 1;
@@ -396,6 +399,47 @@ static void global_row_splits(int B, int H, int L, int* nsplit, int* split_rows)
     const int per = (int)((tiles + want - 1) / want);   // tiles per split
     *split_rows = per * 64;
     *nsplit = (tiles + per - 1) / per;
+}
+
+// Block pattern with the global rows' key splits in the same launch: run length of the block items and number of
+// key splits, chosen together so that runs and splits fill one round of workgroups and end at about the same time.
+// Costs in thousands of cycles, measured on an MI355X: a run pays one set-up (15) and per q tile three steps and
+// the switch to the next q tile (15.6); a split pays one set-up (16) and 2.0 per key tile.  Never more splits than
+// global_row_splits() gives: the workspace size is computed from that.
+static void block_fold_plan(FwdParams* p, int dtype, int D, int B, int H, int L, int* nsplit, int* split_rows) {
+    global_row_splits(B, H, L, nsplit, split_rows);
+    const int64_t bh = (int64_t)B * H;
+    const int64_t entries = (int64_t)p->tiles_per_seq * bh;
+    const int64_t slots = 2 * (int64_t)device_compute_units();
+    const bool runs_ok = dtype != T5A_F32 && (D == 64 || D == 128);
+    if (!runs_ok || getenv("T5A_RUN_LEN") != nullptr || entries + (int64_t)*nsplit * bh <= slots) {
+        choose_runs(p, kBlock, dtype, D, (int64_t)*nsplit * bh);
+        return;
+    }
+    const int tiles = (L + 63) / 64;
+    double best = 0.0;
+    int best_r = 0, best_s = 0;
+    for (int r = 1; r <= 16; ++r) {
+        const int64_t n_runs = (entries + r - 1) / r;
+        const int64_t free_slots = slots - n_runs;
+        if (free_slots < bh) continue;
+        int64_t per_bh = free_slots / bh;
+        if (per_bh > *nsplit) per_bh = *nsplit;
+        if (per_bh < 1) per_bh = 1;
+        const int s_tiles = (int)((tiles + per_bh - 1) / per_bh);
+        const double run_cost = 15.0 + 15.6 * r, split_cost = 16.0 + 2.0 * s_tiles;
+        const double cost = run_cost > split_cost ? run_cost : split_cost;
+        if (best_r == 0 || cost < best) { best = cost; best_r = r; best_s = s_tiles; }
+    }
+    if (best_r == 0) {   // more work than one round holds at any run length
+        choose_runs(p, kBlock, dtype, D, (int64_t)*nsplit * bh);
+        return;
+    }
+    p->run_len = best_r;
+    p->runs_per_seq = p->tiles_per_seq;
+    p->total_items = (int)((entries + best_r - 1) / best_r);
+    *split_rows = best_s * 64;
+    *nsplit = (tiles + best_s - 1) / best_s;
 }
 
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux) {
@@ -470,15 +514,18 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         // (rel = j - i, no end alignment)
         const int nblk = (a->L + a->block_len - 1) / a->block_len;
         p.tiles_per_seq = nblk * ((a->block_len + 127) / 128);
-        choose_runs(&p, kBlock, a->dtype, a->D);
         const int G = a->aux < a->L ? a->aux : a->L;
         const int64_t need = t5a_sparse_workspace_bytes(a->pattern, a->B, a->H, a->L, a->D, a->block_len, a->aux);
-        if (a->aux > 0 && a->workspace != nullptr && need > 0 && G <= 128) {
+        const bool fold = a->aux > 0 && a->workspace != nullptr && need > 0 && G <= 128;
+        int fold_splits = 0, fold_rows = 0;
+        if (fold) block_fold_plan(&p, a->dtype, a->D, a->B, a->H, a->L, &fold_splits, &fold_rows);
+        else choose_runs(&p, kBlock, a->dtype, a->D);
+        if (fold) {
             // one launch: the block items, then the global rows as key splits spread over the whole device; one merge
             if (a->workspace_bytes < need)
                 return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes, %lld needed", (long long)a->workspace_bytes, (long long)need);
             if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
-            global_row_splits(a->B, a->H, a->L, &p.nsplit, &p.split_rows);
+            p.nsplit = fold_splits; p.split_rows = fold_rows;   // (never more splits than the workspace size assumes)
             const int64_t rows = (int64_t)a->B * a->H * p.nsplit * G;
             p.part_o = reinterpret_cast<float*>(a->workspace);
             p.part_l = p.part_o + rows * a->D;

@@ -306,7 +306,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // key tiles form one stream through the LDS rings (the requests for the next q tile's first tiles go out during
     // the last steps of the current one) and the distance LUT is built once per run; a q tile of a sparse pattern
     // is only a few steps long, so that its set-up would otherwise cost as much as its steps.
-    constexpr bool RUNS = MODE == kLocal && G::DMA;
+    constexpr bool RUNS = (MODE == kLocal || MODE == kBlock) && G::DMA;
+    constexpr bool CURSOR = MODE == kLocal && G::DMA;   // one segment: the requests of a run advance cursors
     // head_dim 64, 16-bit types: the Q rows are staged through LDS by LDS-DMA as well (see the prologue)
     constexpr bool QDMA = G::DMA && D == 64;
     // 16-bit inputs, two ways to apply sm_scale * log2(e).  Default: Q is pre-multiplied and rounded back to the
@@ -388,6 +389,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (RUNS) {
         run_next = w * p.run_len;
         run_left = min(p.run_len, p.tiles_per_seq * p.H * p.B - run_next);
+        if (MODE == kBlock && p.nsplit > 1 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
     }
     for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
@@ -574,7 +576,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
     set_qtile(qt);
     if constexpr (RUNS) {
-        if (MODE == kBlock) { seg_nt[0] = (p.aux + BN - 1) / BN; seg_nt[1] = (p.block_len + BN - 1) / BN; }
+        if (MODE == kBlock && gsplit) { seg_nt[0] = (Nseq + BN - 1) / BN; seg_nt[1] = 0; }
+        else if (MODE == kBlock) { seg_nt[0] = (p.aux + BN - 1) / BN; seg_nt[1] = (p.block_len + BN - 1) / BN; }
         else { seg_nt[0] = (BM + 2 * p.block_len - 2 + BN - 1) / BN; seg_nt[1] = nseg > 1 ? (n_side + BN - 1) / BN : 0; }
     } else {
         seg_nt[0] = max(0, seg_end[0] - seg_start[0] + BN - 1) / BN;
@@ -582,7 +585,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     // an even number of tiles per q tile keeps the two score buffers of the pipeline in step from one q tile of a
     // run to the next (the extra tile lies past its segment's end and is skipped)
-    if (RUNS && ((seg_nt[0] + seg_nt[1]) & 1)) {   // (no run-time index: that would move the array to scratch memory)
+    // (the block pattern's q tiles are too short for fast steps anyway: no rounding there)
+    if (RUNS && MODE != kBlock && ((seg_nt[0] + seg_nt[1]) & 1)) {   // (no run-time index: that would move the array to scratch memory)
         if (nseg > 1) seg_nt[1] += 1; else seg_nt[0] += 1;
     }
     const int ntiles = seg_nt[0] + seg_nt[1];   // tiles of one q tile
@@ -650,7 +654,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     int rq_koff[G::SPW], rq_voff[G::SPW];   // this lane's byte offsets inside a tile
 #pragma unroll
     for (int c = 0; c < G::SPW; ++c) rq_koff[c] = rq_voff[c] = 0;
-    if constexpr (RUNS) {
+    if constexpr (CURSOR) {
 #pragma unroll
         for (int c = 0; c < G::SPW; ++c) {
             const int r = (wave * G::SPW + c) * G::RPS + lane / G::LPR, pc = lane % G::LPR;
@@ -661,7 +665,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         rq_q[0] = rq_q[1] = qt;
     }
     auto dma_next = [&](bool is_v, int stage = -1) {
-        if constexpr (RUNS) {
+        if constexpr (CURSOR) {
             const int w = is_v ? 1 : 0;
             const int j0 = w ? rq_j0[1] : rq_j0[0];
             const int q_tile = w ? rq_q[1] : rq_q[0];
@@ -809,7 +813,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                                       : (unsigned)(3 * V_TILE) * ES + (wave - 2) * 4096u;
     if constexpr (QDMA) {
         if constexpr (DENSE) { cursor_seek(0, 0); cursor_dma(0, 0); }
-        else if constexpr (RUNS) { dma_next(false); dma_next(true); }
+        else if constexpr (CURSOR) { dma_next(false); dma_next(true); }
         else { dma_tile(0, false); dma_tile(0, true); }
         const int q_row_bytes = (int)p.q_sr * ES;
         const u32x4 rs = make_rsrc_words(qp, row_end > 0 ? (unsigned)(row_end - 1) * (unsigned)q_row_bytes + D * ES : 0u);
@@ -842,13 +846,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (DMA) {
         if constexpr (QDMA) {
             if constexpr (DENSE) { cursor_dma(1, 1); cursor_dma(2, 2); }   // K1 V1, K2 V2
-            else if constexpr (RUNS) { dma_next(false); dma_next(true); dma_next(false); dma_next(true); }
+            else if constexpr (CURSOR) { dma_next(false); dma_next(true); dma_next(false); dma_next(true); }
             else { dma_tile(1, false); dma_tile(1, true); dma_tile(2, false); dma_tile(2, true); }
         } else if constexpr (DENSE) {
             cursor_seek(0, 0);
             cursor_dma(0, 0); cursor_dma(1, 1); cursor_dma(2, 2);   // K0 V0, K1 V1, K2 V2
             dma_tile(3, false);                                     // K3
-        } else if constexpr (RUNS) {
+        } else if constexpr (CURSOR) {
             for (int i = 0; i < 4; ++i) dma_next(false);
             for (int i = 0; i < 3; ++i) dma_next(true);
         } else {
@@ -1432,7 +1436,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     f32x16 sta[NT], stb[NT];
     fill_classes();
     TileClass tc = classify(0);
-    const bool first_interior = LOCAL && seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+    // q tiles whose tiles all have the same classes: away from the ends of the sequence (local pattern); whole
+    // blocks other than the first, one q tile each, of a sequence without padding (block pattern)
+    auto is_interior = [&]() {
+        if (LOCAL) return seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+        if (MODE == kBlock) return !gsplit && tpb == 1 && blk >= 1 && (blk + 1) * p.block_len <= min(Nseq, n_valid) && i0 + BM <= Mseq;
+        return false;
+    };
+    const bool first_interior = is_interior();
     if constexpr (QDMA) {
         // K0 and V0 landed before the barrier that published the LUT
     } else {
@@ -1457,13 +1468,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (QDMA) wait_vmcnt<3 * G::SPW>();   // K1 has landed; V1 K2 V2 may still be in flight
     __syncthreads();   // the first step overwrites the K buffer this product was read from
     if constexpr (QDMA) {   // K3, into the stage that held the Q rows of two wavefronts
-        if constexpr (RUNS) dma_next(false); else dma_tile(3, false);
+        if constexpr (CURSOR) dma_next(false); else dma_tile(3, false);
     }
 
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         const int kbuf_next = DMA ? (tbase + t + 1) % NSK : (t + 1) & 1;
         const int vbuf = DMA ? (tbase + t) % NSV : t & 1;
-        if constexpr (RUNS) {
+        if constexpr (CURSOR) {
             dma_next(false);
             dma_next(true);
         } else if constexpr (DMA) {
@@ -1561,7 +1572,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
         if constexpr (DENSE) cursor_dma(ST, (ST + 3) & 3);
-        else if constexpr (RUNS) { dma_next(false, ST); dma_next(true, (ST + 3) & 3); }
+        else if constexpr (CURSOR) { dma_next(false, ST); dma_next(true, (ST + 3) & 3); }
         else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
         read_k((ST + 1) & 3, ka);
@@ -1677,7 +1688,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     for (;;) {
         int t = 0;
         while (t < ntiles) {
-            if (DMA && ((tbase + t) & 3) == 0) {
+            if (DMA && ((tbase + t) & 3) == 0 && (t & 1) == 0) {   // (even t: tile t's scores are in sta)
                 // steps t .. t+3 are fast when tiles t .. t+4 are plain: run >= 5.  When the run reaches the
                 // last tile, the final fast step forms an S product for a tile that does not exist (its K
                 // stage holds zeros or a tile of the next q tile) and nobody consumes it, so the run may end
@@ -1737,7 +1748,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             for (int r = 0; r < 16; ++r) cm[r] = 0.f;
             // away from the ends of the sequence every q tile of the local pattern has the same classes
             const bool was_interior = interior;
-            interior = LOCAL && seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
+            interior = is_interior();
             if (!(interior && was_interior)) fill_classes();
             tc = classify(0);
             if (tc.side != 0) refill_cm(tc.side);
