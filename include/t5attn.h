@@ -84,14 +84,24 @@ typedef struct t5a_bias {
     int64_t stride_bucket;        /* elements between buckets (torch stride(0)) */
     int64_t stride_head;          /* elements between heads   (torch stride(1)) */
     void* lut; int64_t lut_bytes;
+    /* 0: lut holds the plain images (t5a_bias_lut_bytes).  w > 0: it holds the images with the sliding window
+     * |rel| < w folded in (t5a_bias_lut_bytes_windowed), which only t5a_fwd_sparse(T5A_PATTERN_LOCAL) with
+     * block_len == w fetches; every other call rejects such a buffer.  A plain buffer handed to the local pattern is
+     * ignored (its work items fill their LUTs themselves, 8 % of its run time at L=16384). */
+    int32_t lut_window;
+    int32_t reserved;
 } t5a_bias;
 /* 0 when the kernels cannot use a LUT buffer for these parameters (very large max_distance); causal selects
  * the unidirectional buckets, as in t5a_fwd_dense. */
 int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t causal);
+/* Size of a buffer for the images with the window |rel| < window folded in (bidirectional buckets; see
+ * t5a_bias.lut_window); 0 when the local pattern cannot use one for this window.  No counterpart in the reference,
+ * whose local attention materialises bias and mask per call (src/turbot5/model/attentions.py:598-618). */
+int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t window);
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 109
+#define T5A_ABI_VERSION 110
 int t5a_version(void);
 const char* t5a_last_error(void);
 

@@ -291,3 +291,84 @@ def test_local_with_padding_on_either_side(gpu_device, dtype, L, Bl):
     assert torch.isfinite(out[valid[:, None, :].expand(B, H, L)]).all()
     err = (out - want).abs()[valid[:, None, :, None].expand(B, H, L, D)].max().item()
     assert err <= TOL[dtype], err
+
+
+@pytest.mark.parametrize("L,Bl", [(1024, 128), (700, 64), (512, 32)])
+def test_local_windowed_lut_buffer_gives_identical_results(gpu_device, L, Bl):
+    """The local pattern's LUT images (sliding window folded in), built once into a buffer and fetched by later
+    launches, are the images its work items otherwise fill for themselves: outputs are bit-identical without the
+    buffer, on the launch that builds it and on those that find it ready; buffers for different windows and the plain
+    one of the same table are separate entries."""
+    from turbot5_amd import ops
+    B, H, D = 2, 3, 64
+    q, k, v = (rnd(B, H, L, D, seed=140 + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+    table = rnd(32, H, seed=143, scale=1.0).to(gpu_device)
+    run = lambda bl=Bl: ops.local_attention_with_fusing_bias(q, k, v, table, bl).cpu()  # noqa: E731
+    ops.clear_bias_luts()
+    ops.BIAS_LUT_CACHE = False
+    try:
+        plain = run()
+        other_plain = run(2 * Bl)
+        dense_plain = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0).cpu()
+    finally:
+        ops.BIAS_LUT_CACHE = True
+    assert len(ops._BIAS_LUTS) == 0
+    first, second = run(), run()
+    assert len(ops._BIAS_LUTS) == 1
+    assert torch.equal(plain.view(torch.int16), first.view(torch.int16))
+    assert torch.equal(plain.view(torch.int16), second.view(torch.int16))
+    other = run(2 * Bl)                # another window: its own images
+    dense = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0).cpu()   # the plain ones
+    from turbot5_amd import _lib
+    has_other = _lib.load().t5a_bias_lut_bytes_windowed(H, 32, 128, 2 * Bl) > 0   # (a window of 256 is too long to fetch)
+    assert len(ops._BIAS_LUTS) == (3 if has_other else 2)
+    assert torch.equal(other_plain.view(torch.int16), other.view(torch.int16))
+    assert torch.equal(dense_plain.view(torch.int16), dense.view(torch.int16))
+    assert torch.equal(plain.view(torch.int16), run().view(torch.int16))
+    want = O.local_attention_blocked(q.cpu(), k.cpu(), v.cpu(), table.cpu(), Bl) if L % Bl == 0 else None
+    if want is not None:
+        assert (first.float() - want).abs().max().item() <= 2e-2
+    ops.clear_bias_luts()
+
+
+def test_windowed_lut_buffer_is_only_for_its_window(gpu_device):
+    """A buffer of windowed images is refused by every call that would read it as something else; a plain buffer
+    handed to the local pattern is ignored."""
+    import ctypes as C
+    from turbot5_amd import _lib as lib_mod, ops
+    lib = lib_mod.load()
+    B, H, L, D, Bl = 1, 2, 256, 64, 64
+    q, k, v = (rnd(B, H, L, D, seed=150 + i, dtype=torch.bfloat16).to(gpu_device) for i in range(3))
+    table = rnd(32, H, seed=153, scale=1.0).to(gpu_device)
+    o = torch.empty_like(q)
+    nbytes = lib.t5a_bias_lut_bytes_windowed(H, 32, 128, Bl)
+    assert nbytes > 0
+    lut = torch.zeros(nbytes, dtype=torch.uint8, device=gpu_device)
+
+    def sparse_args(block_len, window):
+        a = lib_mod.T5ASparseArgs()
+        a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+        for name, t in (("q_strides", q), ("k_strides", k), ("v_strides", v), ("o_strides", o)):
+            setattr(a, name, (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2)))
+        a.dtype, a.B, a.H, a.L, a.D = lib_mod.T5A_BF16, B, H, L, D
+        a.pattern, a.block_len, a.aux, a.sm_scale = lib_mod.PATTERN_LOCAL, block_len, 0, 1.0
+        a.bias.table, a.bias.table_dtype = table.data_ptr(), lib_mod.T5A_F32
+        a.bias.num_buckets, a.bias.max_distance = 32, 128
+        a.bias.stride_bucket, a.bias.stride_head = table.stride(0), table.stride(1)
+        a.bias.lut, a.bias.lut_bytes, a.bias.lut_window, a.bias.lut_ready = lut.data_ptr(), nbytes, window, 0
+        return a
+
+    stream = ops._stream(q)
+    with torch.cuda.device(gpu_device):
+        assert lib.t5a_fwd_sparse(C.byref(sparse_args(Bl, Bl)), stream) == 0           # builds and uses it
+        built = o.clone()
+        assert lib.t5a_fwd_sparse(C.byref(sparse_args(2 * Bl, Bl)), stream) != 0       # another window: refused
+        assert b"window" in lib.t5a_last_error()
+        a = sparse_args(Bl, 0)                                                         # declared plain: ignored
+        a.bias.lut_ready = 1
+        o.zero_()
+        assert lib.t5a_fwd_sparse(C.byref(a), stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(o.view(torch.int16), built.view(torch.int16))
+        a = sparse_args(Bl, -3)
+        assert lib.t5a_fwd_sparse(C.byref(a), stream) != 0

@@ -32,7 +32,7 @@ def test_header_symbols_are_exported(lib):
 
 def test_struct_sizes_follow_the_header(lib):
     # natural alignment, no packing: catches a field added on one side only
-    assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8
+    assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8 + 2 * 4
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 2 * 8
@@ -109,6 +109,15 @@ def test_workspace_sizes_and_checks_without_gpu(lib):
     assert handle.t5a_bias_lut_bytes(12, 32, 4096, 0) == 0      # too long for the kernel's fetch: not offered
     assert handle.t5a_bias_lut_bytes(0, 32, 128, 0) == 0
     assert handle.t5a_bias_lut_bytes(12, 3, 128, 0) == 0        # bad bucket parameters
+    # ... with a sliding window folded in: the image reaches 96 entries past the window when that is wider than the
+    # buckets' saturation distance (91 for 32 / 128), and is the plain one's size otherwise
+    for window, sat in ((128, 128), (64, 91), (32, 91)):
+        quads = (2 * (sat + 96) + 1 + 6) // 4 + 1
+        quads += (4 - quads) % 16
+        assert handle.t5a_bias_lut_bytes_windowed(12, 32, 128, window) == 12 * 4 * (4 * quads) * 4
+    assert handle.t5a_bias_lut_bytes_windowed(12, 32, 128, 256) == 0     # too long for the kernel's fetch
+    assert handle.t5a_bias_lut_bytes_windowed(12, 32, 128, 0) == 0
+    assert handle.t5a_bias_lut_bytes_windowed(12, 32, 128, 300) == 0     # wider than the windows that go into the LUT
     # launch plan of a packed batch: 64 bytes of counts, 8 lists of 2 * ceil(items / 8) entries of 32 bytes,
     # 16 bytes per item for spilled entries; items = (total_q / 128 + B) * H
     items = (70000 // 128 + 32) * 12

@@ -13,13 +13,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 109   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 110   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
-    "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes",
+    "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes", "t5a_bias_lut_bytes_windowed",
     "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
     "t5a_rmsnorm",
 )
@@ -29,7 +29,8 @@ class T5ABias(C.Structure):
     _fields_ = [("table", C.c_void_p), ("table_dtype", C.c_int32), ("num_buckets", C.c_int32),
                 ("max_distance", C.c_int32), ("lut_ready", C.c_int32),
                 ("stride_bucket", C.c_int64), ("stride_head", C.c_int64),
-                ("lut", C.c_void_p), ("lut_bytes", C.c_int64)]
+                ("lut", C.c_void_p), ("lut_bytes", C.c_int64),
+                ("lut_window", C.c_int32), ("reserved", C.c_int32)]
 
 
 class T5ADenseArgs(C.Structure):
@@ -130,6 +131,8 @@ def load() -> C.CDLL:
         lib.t5a_rmsnorm.restype = C.c_int
         lib.t5a_bias_lut_bytes.argtypes = [C.c_int32] * 4
         lib.t5a_bias_lut_bytes.restype = C.c_int64
+        lib.t5a_bias_lut_bytes_windowed.argtypes = [C.c_int32] * 4
+        lib.t5a_bias_lut_bytes_windowed.restype = C.c_int64
         lib.t5a_varlen_workspace_bytes.argtypes = [C.c_int32] * 3
         lib.t5a_varlen_workspace_bytes.restype = C.c_int64
         lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7

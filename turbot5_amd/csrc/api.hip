@@ -140,19 +140,27 @@ static int fill_bias(const t5a_bias& b, bool bidirectional, FwdParams* p) {
 }
 
 // Optional buffer with the distance LUTs of all heads: checked, built on the first use, handed to the kernel.
-static int prepare_lut(const t5a_bias& b, bool causal, hipStream_t stream, FwdParams* p) {
+// window: 0, or the sliding window of the local pattern when it is folded into the LUT
+static int prepare_lut(const t5a_bias& b, bool causal, hipStream_t stream, FwdParams* p, int window = 0) {
     if (b.table == nullptr || b.lut == nullptr) return T5A_OK;
-    const int64_t need = bias_lut_bytes(p->H, p->bs, causal);
+    if (b.lut_window < 0) return fail(T5A_ERR_SHAPE, "bias.lut_window %d", b.lut_window);
+    if (b.lut_window != window) {
+        if (b.lut_window == 0) return T5A_OK;   // plain images, windowed ones wanted: the kernel fills its LUTs itself
+        return fail(T5A_ERR_PATTERN, "bias.lut holds the images for the window %d: only the local pattern with that block_len reads them",
+                    b.lut_window);
+    }
+    const int64_t need = bias_lut_bytes(p->H, p->bs, causal, window);
     if (need == 0) return T5A_OK;   // not usable for these parameters: the kernel builds its LUTs itself
     if (b.lut_bytes < need)
         return fail(T5A_ERR_WORKSPACE, "bias.lut too small: %lld bytes, t5a_bias_lut_bytes() asks for %lld",
                     (long long)b.lut_bytes, (long long)need);
     if ((reinterpret_cast<uintptr_t>(b.lut) & 15) != 0) return fail(T5A_ERR_STRIDE, "bias.lut must be 16-byte aligned");
     if (b.lut_ready == 0) {
-        hipError_t e = launch_bias_lut(*p, causal, static_cast<float*>(b.lut), stream);
+        hipError_t e = launch_bias_lut(*p, causal, static_cast<float*>(b.lut), stream, window);
         if (e != hipSuccess) return fail(T5A_ERR_LAUNCH, "bias LUT build: %s", hipGetErrorString(e));
     }
     p->lut_global = static_cast<const float*>(b.lut);
+    p->lut_window = window;
     return T5A_OK;
 }
 
@@ -185,6 +193,12 @@ int64_t t5a_bias_lut_bytes(int32_t H, int32_t num_buckets, int32_t max_distance,
     BucketSpec bs;
     if (H <= 0 || make_bucket_spec(causal == 0, num_buckets, max_distance, &bs) != T5A_OK) return 0;
     return bias_lut_bytes(H, bs, causal != 0);
+}
+
+int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_distance, int32_t window) {
+    BucketSpec bs;
+    if (H <= 0 || window <= 0 || window > kMaxLutWindow || make_bucket_spec(true, num_buckets, max_distance, &bs) != T5A_OK) return 0;
+    return bias_lut_bytes(H, bs, false, window);
 }
 
 int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t* out) {
@@ -499,7 +513,8 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.exact_scale = a->exact_scores != 0;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if ((rc = prepare_lut(a->bias, false, s, &p))) return rc;
+    const bool window_in_lut = a->pattern == T5A_PATTERN_LOCAL && a->block_len <= kMaxLutWindow;
+    if ((rc = prepare_lut(a->bias, false, s, &p, window_in_lut ? a->block_len : 0))) return rc;
 
     if (a->pattern == T5A_PATTERN_BLOCK) {
         if (a->L < a->block_len) {

@@ -788,8 +788,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // register written by a load issued from inline assembly is still in flight and may copy it too early.
     const int nbt = p.bs.bidirectional ? 2 * p.bs.nb : p.bs.nb;
     const bool col_in_lanes = nbt <= 64;
-    // (a per-table buffer holds the plain LUTs: not the ones with a window folded in)
-    const bool lut_cached = has_bias && p.lut_global != nullptr && !win_lut;   // the host checked qlen <= 512
+    // (the host checked qlen <= 512, and that a buffer of windowed images goes with this window)
+    const bool lut_cached = has_bias && p.lut_global != nullptr && (win_lut ? p.lut_window == p.block_len : p.lut_window == 0);
     const int col_esize = p.table_dtype == T5A_F32 ? 4 : 2;
     // byte offset of this lane's bucket in the table, from the 4-byte aligned address at or below its start
     const unsigned col_misalign = (unsigned)(reinterpret_cast<uintptr_t>(p.table) & 3);

@@ -61,6 +61,7 @@ struct FwdParams {
     int exact_scale;     // 16-bit inputs: apply c1 to the fp32 product instead of to Q (see attn_fwd.hip)
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;
     const float* lut_global;   // optional: the distance LUTs of all heads, (H, 4, qlen) floats (lut.hip)
+    int lut_window;            // 0: plain images; w: images with the window |rel| < w folded in (local pattern)
     int block_len, aux, n_side;
     int align_end;       // 1: query i sits at key position i + N - M (KV-cache alignment); 0: at i
     // key split (dense, unpacked, align_end == 0): split s of nsplit covers keys [s*split_rows, (s+1)*split_rows)
@@ -78,8 +79,8 @@ int fail(int code, const char* fmt, ...);
 int make_bucket_spec(bool bidirectional, int num_buckets, int max_distance, BucketSpec* out);
 
 // distance LUTs of all heads in a caller-provided buffer (lut.hip)
-int64_t bias_lut_bytes(int H, const BucketSpec& bs, bool causal);
-hipError_t launch_bias_lut(const FwdParams& p, bool causal, float* out, hipStream_t stream);
+int64_t bias_lut_bytes(int H, const BucketSpec& bs, bool causal, int window = 0);
+hipError_t launch_bias_lut(const FwdParams& p, bool causal, float* out, hipStream_t stream, int window = 0);
 
 // launchers (attn_fwd.hip, splitk.hip)
 hipError_t launch_fwd_bf16(const FwdParams& p, int D, int mode, bool causal, hipStream_t stream);

@@ -68,16 +68,19 @@ _BIAS_LUTS: "OrderedDict[tuple, tuple]" = OrderedDict()
 BIAS_LUT_CACHE = True
 
 
-def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int, causal: bool, ref: torch.Tensor):
-    """-> (lut buffer or None, cache key to commit after a successful launch or None)."""
+def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int, causal: bool, ref: torch.Tensor,
+              window: int = 0):
+    """-> (lut buffer or None, cache key to commit after a successful launch or None).
+    window > 0: the images with that sliding window folded in (what the local pattern's work items fetch)."""
     if not BIAS_LUT_CACHE or torch.cuda.is_current_stream_capturing():
         return None, None   # a build recorded into a graph would not have run when the next eager launch reads it
     key = (bias.data_ptr(), bias._version, bias.stride(0), bias.stride(1), bias.dtype, H, num_buckets, max_distance,
-           bool(causal), ref.device.index, _stream(ref))
+           bool(causal), ref.device.index, _stream(ref), int(window))
     hit = _BIAS_LUTS.get(key)
     pending = None
     if hit is None:
-        nbytes = L.load().t5a_bias_lut_bytes(H, num_buckets, max_distance, int(bool(causal)))
+        nbytes = (L.load().t5a_bias_lut_bytes_windowed(H, num_buckets, max_distance, int(window)) if window > 0
+                  else L.load().t5a_bias_lut_bytes(H, num_buckets, max_distance, int(bool(causal))))
         if nbytes <= 0:
             return None, None
         lut = torch.empty(nbytes, device=ref.device, dtype=torch.uint8)
@@ -86,7 +89,7 @@ def _bias_lut(b, bias: torch.Tensor, H: int, num_buckets: int, max_distance: int
     else:
         lut = hit[1]
         b.lut_ready = 1
-    b.lut, b.lut_bytes = lut.data_ptr(), lut.numel()
+    b.lut, b.lut_bytes, b.lut_window = lut.data_ptr(), lut.numel(), int(window)
     return lut, pending
 
 
@@ -109,7 +112,7 @@ def clear_bias_luts():
 
 
 def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_distance: int, ref: torch.Tensor,
-                 causal: bool = False):
+                 causal: bool = False, window: int = 0):
     b = L.T5ABias()
     if bias is None:
         b.table = None
@@ -127,7 +130,7 @@ def _bias_struct(bias: Optional[torch.Tensor], H: int, num_buckets: int, max_dis
     b.max_distance = max_distance
     b.stride_bucket = table.stride(0)
     b.stride_head = table.stride(1)
-    lut, pending = (_bias_lut(b, bias, H, num_buckets, max_distance, causal, ref)
+    lut, pending = (_bias_lut(b, bias, H, num_buckets, max_distance, causal, ref, window)
                     if table.data_ptr() == bias.data_ptr() else (None, None))
     return b, (table, lut, pending, bias)   # alive until the launch has been queued; see _commit_lut
 
@@ -352,7 +355,9 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
         a.seq_lens = seq_lens.data_ptr()
     if seq_starts is not None:
         a.seq_starts = seq_starts.data_ptr()
-    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q)
+    # the local pattern's work items fetch LUT images that have the window folded in (windows up to 256)
+    window = int(block_len) if pattern == L.PATTERN_LOCAL and int(block_len) <= 256 else 0
+    a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, window=window)
     lib = L.load()
     ws_bytes = lib.t5a_sparse_workspace_bytes(pattern, B, H, Lq, D, int(block_len), int(aux))
     workspace = None
