@@ -612,11 +612,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto tile_of = [&](int t, int& sg, int& j0) {
         if constexpr (RUNS) {
             int ahead = 0;
+            if (t >= ntiles) { t -= ntiles; ++ahead; }          // (requests run at most four tiles ahead: two q tiles
+            if (t >= ntiles) { t -= ntiles; ++ahead; }          // further on at the very most, with q tiles of 2+ tiles)
             while (t >= ntiles) { t -= ntiles; ++ahead; }
             const int q_tile = qt + ahead;
             sg = t >= seg_nt[0] ? 1 : 0;
             const int ts = t - (sg ? seg_nt[0] : 0);
-            if (MODE == kBlock) j0 = sg ? (q_tile / tpb) * p.block_len + ts * BN : ts * BN;
+            // (a scalar division costs some forty instructions, and this runs for every request)
+            if (MODE == kBlock) j0 = sg ? (tpb == 1 ? q_tile : q_tile / tpb) * p.block_len + ts * BN : ts * BN;
             else j0 = sg ? ts * BN : q_tile * BM - p.block_len + 1 + ts * BN;
             return q_tile < qt_last;
         } else {
@@ -725,6 +728,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
     };
     // ---------------------------------------------------------------- Q fragments: loads first
+    int wq_lo[2] = {0, 0}, wq_hi[2] = {0, 0}, lq_pos[2] = {0, 0};   // query positions per segment, see set_positions
     int iw0 = i0 + wave * 32;      // first row of this wavefront
     int iw1 = iw0 + 31;
     int irow = iw0 + lr;           // this lane's query row
@@ -1040,10 +1044,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         tile_of(t, c.sg, c.j0);
         const int kind = (c.sg ? seg_kind[1] : seg_kind[0]);
         const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
-        int qlo, qhi;
-        if (kind == 0) { qlo = iw0 + P; qhi = iw1 + P; }
-        else if (kind == 1) { qlo = iw0 % p.block_len + p.aux; qhi = qlo + 31; }
-        else { qlo = min(iw0 / p.aux, n_side - 1); qhi = min(iw1 / p.aux, n_side - 1); }
+        (void)kind;
+        constexpr bool cached = MODE == kBlock || MODE == kTGlobal;   // positions kept per q tile (set_positions)
+        const int qlo = cached ? (c.sg ? wq_lo[1] : wq_lo[0]) : iw0 + P, qhi = cached ? (c.sg ? wq_hi[1] : wq_hi[0]) : iw1 + P;
         const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
         c.skip = iw0 >= row_end;                              // wavefront without live rows
         if (CAUSAL) c.skip = c.skip || rel_min > 0;           // every key is in the future of every row
@@ -1129,12 +1132,30 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
 #pragma unroll
     for (int r = 0; r < 16; ++r) cm[r] = 0.f;
 
-    auto lane_qpos = [&](int sg) {   // this lane's query position in the segment's bias geometry
-        const int kind = (sg ? seg_kind[1] : seg_kind[0]);
+    // Query positions in each segment's bias geometry, once per q tile (they take integer divisions by run-time
+    // values, some forty instructions each: not something for every tile): the wavefront's range and this lane's own.
+    auto position_of = [&](int kind, int row) {
+        if (kind == 0) return row + P;
+        if (kind == 1) return row % p.block_len + p.aux;
+        return min(row / p.aux, n_side - 1);   // trailing tokens past the last full block join it
+    };
+    constexpr bool POS_CACHE = MODE == kBlock || MODE == kTGlobal;   // (the other patterns' positions are row + P)
+    auto set_positions = [&]() {
+        if constexpr (!POS_CACHE) return;
         const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
-        if (kind == 0) return ir + P;
-        if (kind == 1) return ir % p.block_len + p.aux;
-        return min(ir / p.aux, n_side - 1);   // trailing tokens past the last full block join it
+        lq_pos[0] = position_of(seg_kind[0], ir);
+        wq_lo[0] = position_of(seg_kind[0], iw0);
+        wq_hi[0] = seg_kind[0] == 1 ? wq_lo[0] + 31 : position_of(seg_kind[0], iw1);
+        if (nseg > 1) {
+            lq_pos[1] = position_of(seg_kind[1], ir);
+            wq_lo[1] = position_of(seg_kind[1], iw0);
+            wq_hi[1] = seg_kind[1] == 1 ? wq_lo[1] + 31 : position_of(seg_kind[1], iw1);
+        }
+    };
+    set_positions();
+    auto lane_qpos = [&](int sg) {
+        if constexpr (POS_CACHE) return sg ? lq_pos[1] : lq_pos[0];
+        else return min(irow, max(row_end - 1, iw0)) + P;
     };
 
     // K fragments of one tile (16-bit types): issued early so that the LDS latency hides behind
@@ -1731,6 +1752,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             tbase += ntiles;
             set_qtile(qt);
             iw0 = i0 + wave * 32; iw1 = iw0 + 31; irow = iw0 + lr; row_ok = irow < row_end;
+            set_positions();
             prefetch_q(qt + 1);
             if (!exact) {
 #pragma unroll
