@@ -101,7 +101,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 110
+#define T5A_ABI_VERSION 111
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -207,6 +207,15 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           [G global tokens | own block] is masked iff token b * block_len + c is padding, the last G
  *           columns never (always in block 0); the first G rows attend every key, padding included
  *           (:788-800).
+ * key_bits (optional, LOCAL and BLOCK; instead of seq_lens / seq_starts): validity of every token as a bit set,
+ * for attention masks of any shape (holes, padding on either side).  (B, key_bits_stride) uint32 words on the
+ * device; token j of sequence b is bit (j & 31) of word 8 + (j >> 5) -- eight zero words in front, and zero words
+ * behind the last token up to at least t5a_sparse_key_bits_words(L, block_len, aux) words in all.
+ *   LOCAL   keys whose bit is 0 are not attended (the key half of the reference's local mask,
+ *           src/turbot5/model/utils.py:174-188).
+ *   BLOCK   the reference's additive mask as it lays it out (attentions.py:722-732), for any mask: list column
+ *           c < block_len of [G global tokens | own block] is masked iff token b * block_len + c has bit 0, the
+ *           last G columns never (always in block 0); the first G rows attend every key.
  * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
  * the G global rows, which attend all L keys, are computed as key splits spread over the whole
  * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
@@ -224,7 +233,11 @@ typedef struct t5a_sparse_args {
     t5a_bias bias;
     const int32_t* seq_lens;
     const int32_t* seq_starts;
+    const uint32_t* key_bits;
+    int64_t key_bits_stride;      /* words per sequence */
 } t5a_sparse_args;
+/* words per sequence that key_bits needs (front padding, ceil(L / 32), back padding) */
+int64_t t5a_sparse_key_bits_words(int32_t L, int32_t block_len, int32_t aux);
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux);
 int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);
 

@@ -64,12 +64,16 @@ def test_attention_module_output_tuple(gpu_device):
     mask = torch.ones(2, 96, device=gpu_device)
     mask[1, 50:] = 0
     mask[0, :3] = 0
-    with pytest.raises(NotImplementedError):         # left padding: local and transient-global only
-        T5ATTENTION_TYPES["block"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
-    mask[1, 20:30] = 0
-    for name in ("local", "block", "transient-global"):       # holes
-        with pytest.raises(NotImplementedError):
-            T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
+    with torch.no_grad():                            # left padding: every pattern
+        for name in ("local", "block", "transient-global"):
+            out = T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device).eval()(x, mask=mask)
+            assert torch.isfinite(out[0][mask.bool()]).all()
+        mask[1, 20:30] = 0                           # holes: local and block (validity bit sets)
+        for name in ("local", "block"):
+            out = T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device).eval()(x, mask=mask)
+            assert torch.isfinite(out[0][mask.bool()]).all()
+    with pytest.raises(NotImplementedError):
+        T5ATTENTION_TYPES["transient-global"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
 
 
 def test_flash_encoder_with_padding(gpu_device):
@@ -297,10 +301,14 @@ def test_local_encoder_with_right_padding(gpu_device):
     with torch.no_grad():
         got = m(ids.to(gpu_device), left.to(gpu_device)).cpu()
     assert (got[left.bool()] - want[left.bool()]).abs().max().item() <= 2e-3
-    holes = torch.ones(3, 256)
+    holes = torch.ones(3, 256)     # masks with holes: the keys' validity as bit sets
     holes[1, 40:50] = 0
-    with pytest.raises(NotImplementedError), torch.no_grad():
-        m(ids.to(gpu_device), holes.to(gpu_device))
+    holes[2, ::7] = 0
+    holes[2, :20] = 0
+    want = OM.encoder_forward(sd, cfg, ids, holes, attention_type="local")
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), holes.to(gpu_device)).cpu()
+    assert (got[holes.bool()] - want[holes.bool()]).abs().max().item() <= 2e-3
 
 
 def test_transient_global_encoder_with_right_padding(gpu_device):
@@ -347,10 +355,15 @@ def test_block_encoder_with_right_padding(gpu_device):
         got = m(ids.to(gpu_device), mask.to(gpu_device)).cpu()
     valid = mask.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
-    left = torch.ones(4, 256)
-    left[1, :10] = 0
-    with pytest.raises(NotImplementedError), torch.no_grad():
-        m(ids.to(gpu_device), left.to(gpu_device))
+    other = torch.ones(4, 256)     # left padding and holes: validity bit sets
+    other[1, :10] = 0
+    other[2, 100:140] = 0
+    other[3, ::5] = 0
+    want = OM.encoder_forward(sd, cfg, ids, other, attention_type="block")
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), other.to(gpu_device)).cpu()
+    valid = other.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 2e-3
 
 
 @pytest.mark.parametrize("attention_dtype", [None, torch.bfloat16])

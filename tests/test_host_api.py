@@ -35,7 +35,7 @@ def test_struct_sizes_follow_the_header(lib):
     assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8 + 2 * 4
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
-    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 2 * 8
+    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 4 * 8
     assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4 + 2 * 8
     assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 5 * 8
 

@@ -13,14 +13,14 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 110   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 111   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
     "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes", "t5a_bias_lut_bytes_windowed",
-    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
+    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_sparse_key_bits_words", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
     "t5a_rmsnorm",
 )
 
@@ -66,7 +66,8 @@ class T5ASparseArgs(C.Structure):
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("L", C.c_int32), ("D", C.c_int32),
                 ("pattern", C.c_int32), ("block_len", C.c_int32), ("aux", C.c_int32), ("n_side", C.c_int32),
                 ("sm_scale", C.c_float), ("exact_scores", C.c_int32),
-                ("bias", T5ABias), ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p)]
+                ("bias", T5ABias), ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p),
+                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64)]
 
 
 class T5ASplitKArgs(C.Structure):
@@ -137,6 +138,8 @@ def load() -> C.CDLL:
         lib.t5a_varlen_workspace_bytes.restype = C.c_int64
         lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7
         lib.t5a_sparse_workspace_bytes.restype = C.c_int64
+        lib.t5a_sparse_key_bits_words.argtypes = [C.c_int32] * 3
+        lib.t5a_sparse_key_bits_words.restype = C.c_int64
         _lib = lib
     return _lib
 

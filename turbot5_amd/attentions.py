@@ -352,10 +352,22 @@ class T5FlashAttention(_T5AttentionBase):
 
 
 class _SparseBase(_T5AttentionBase):
-    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions, left_padding_ok=True):
+    def _key_bits(self, mask, block_len, aux=0):
+        """Validity bit sets of a mask of any shape (ops.pack_key_bits), kept with the mask's other derived data."""
+        _, unpad = _mask_info(mask)
+        plans = unpad[2]
+        key = ("key_bits", int(block_len), int(aux))
+        bits = plans.get(key)
+        if bits is None:
+            bits = plans[key] = ops.pack_key_bits(mask, block_len, aux)
+        return bits
+
+    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions, left_padding_ok=True,
+                    bits_ok=False):
         """-> (lengths, first rows): (B,) int32 device tensors for a batch whose rows are each ONE run of valid
         tokens (padding on the right, and on the left where the pattern takes it); (None, None) for all ones.
-        First rows are None for right padding."""
+        First rows are None for right padding.  ``bits_ok``: any other mask gives ("bits", None) -- the caller passes
+        validity bit sets instead."""
         if past_key_value is not None:
             warnings.warn('Currently, passing past key value states is not supported.')
         if use_cache is not None:
@@ -375,6 +387,8 @@ class _SparseBase(_T5AttentionBase):
                             starts = plans["starts"] = (unpad[1][1][:B] - torch.arange(
                                 B, device=mask.device, dtype=torch.int32) * L).contiguous()
                         return unpad[1][0], starts
+                if bits_ok:
+                    return "bits", None
                 raise NotImplementedError(
                     f"{type(self).__name__} runs as tile skipping for attention masks whose rows are one run of valid "
                     "tokens (padding on the right" + (" or on the left" if left_padding_ok else "")
@@ -403,15 +417,19 @@ class T5LocalAttention(_SparseBase):
                 use_cache=None, output_attentions=False):
         # right-padded batches: the keys of a sequence end at its length (the key half of the reference's
         # local mask, utils.py:174-188); outputs at padded positions mean nothing, as in the reference
-        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
+        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
+                                                bits_ok=True)
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
         # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
         block_len = min(self.block_len, hidden_states.shape[1])
+        key_bits = None
+        if isinstance(seq_lens, str):   # a mask with holes: the keys' validity as bit sets
+            seq_lens, key_bits = None, self._key_bits(mask, block_len)
         out = ops.local_attention_with_fusing_bias(
             q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
             self.relative_attention_max_distance, seq_lens=seq_lens, seq_starts=seq_starts,
-            exact_scores=self._exact)
+            exact_scores=self._exact, key_bits=key_bits)
         return self._finish(out, hidden_states, table)
 
 
@@ -426,15 +444,19 @@ class T5BlockAttention(_SparseBase):
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
         # right-padded batches: the reference's additive mask over its key list (attentions.py:722-732)
+        # (left padding and holes: validity bit sets, looked up per tile)
         seq_lens, _ = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                                       left_padding_ok=False)
+                                       left_padding_ok=False, bits_ok=True)
         if seq_lens is not None and hidden_states.shape[1] < self.block_len:
             raise NotImplementedError("T5BlockAttention: padded batches shorter than one block are not supported")
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
+        key_bits = None
+        if isinstance(seq_lens, str):
+            seq_lens, key_bits = None, self._key_bits(mask, self.block_len, self.n_global_tokens)
         out = ops.block_attention_with_fusing_bias(
             q, k, v, table, self.block_len, self.n_global_tokens, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance, exact_scores=self._exact, seq_lens=seq_lens)
+            self.relative_attention_max_distance, exact_scores=self._exact, seq_lens=seq_lens, key_bits=key_bits)
         return self._finish(out, hidden_states, table)
 
 

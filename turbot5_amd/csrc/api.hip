@@ -456,6 +456,12 @@ static void block_fold_plan(FwdParams* p, int dtype, int D, int B, int H, int L,
     *nsplit = (tiles + best_s - 1) / best_s;
 }
 
+int64_t t5a_sparse_key_bits_words(int32_t L, int32_t block_len, int32_t aux) {
+    if (L < 0 || block_len <= 0 || aux < 0) return -1;
+    // tiles reach up to block_len + 128 keys past the last token, the block pattern looks block_len + aux further
+    return kKeyBitsFront + ((int64_t)L + 2 * (int64_t)block_len + aux + 256 + 31) / 32 + 4;
+}
+
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux) {
     if (B < 0 || H < 0 || L < 0 || D < 0 || block_len <= 0 || aux < 0) return -1;
     if (pattern != T5A_PATTERN_BLOCK || aux == 0 || L < block_len) return 0;
@@ -508,12 +514,25 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         return fail(T5A_ERR_PATTERN, "seq_starts needs seq_lens and the local or transient-global pattern");
     p.len_k = a->seq_lens;
     p.start_k = a->seq_starts;
+    if (a->key_bits != nullptr) {
+        if (a->pattern == T5A_PATTERN_TGLOBAL) return fail(T5A_ERR_PATTERN, "key_bits is for the local and block patterns");
+        if (a->seq_lens != nullptr) return fail(T5A_ERR_PATTERN, "key_bits and seq_lens are alternatives");
+        const int64_t need = t5a_sparse_key_bits_words(a->L, a->block_len, a->aux);
+        if (a->key_bits_stride < need)
+            return fail(T5A_ERR_SHAPE, "key_bits_stride %lld, t5a_sparse_key_bits_words() asks for %lld",
+                        (long long)a->key_bits_stride, (long long)need);
+        if ((reinterpret_cast<uintptr_t>(a->key_bits) & 3) != 0) return fail(T5A_ERR_STRIDE, "key_bits must be 4-byte aligned");
+        if (a->pattern == T5A_PATTERN_BLOCK && a->L < a->block_len)
+            return fail(T5A_ERR_PATTERN, "block pattern: key_bits with a sequence shorter than one block is not supported");
+        p.key_bits = a->key_bits;
+        p.key_bits_stride = a->key_bits_stride;
+    }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
     p.c1 = a->sm_scale * kLog2e;
     p.exact_scale = a->exact_scores != 0;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;
     hipStream_t s = (hipStream_t)stream;
-    const bool window_in_lut = a->pattern == T5A_PATTERN_LOCAL && a->block_len <= kMaxLutWindow;
+    const bool window_in_lut = a->pattern == T5A_PATTERN_LOCAL && a->block_len <= kMaxLutWindow && a->key_bits == nullptr;
     if ((rc = prepare_lut(a->bias, false, s, &p, window_in_lut ? a->block_len : 0))) return rc;
 
     if (a->pattern == T5A_PATTERN_BLOCK) {
@@ -564,6 +583,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         FwdParams g = p;
         g.run_len = 1;
         g.len_k = nullptr;
+        g.key_bits = nullptr;
         g.M = G;
         g.N = a->L;
         g.tiles_per_seq = (g.M + 127) / 128;
@@ -594,7 +614,9 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         return finish(launch_fwd(g, a->dtype, a->D, kDense, false, s), "t5a_fwd_sparse(block, global rows)");
     }
     p.tiles_per_seq = (a->L + 127) / 128;
-    const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? kTGlobal : (a->block_len <= kMaxLutWindow ? kLocal : kLocalWide);
+    // (validity bit sets go with the instantiation that masks per element)
+    const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? kTGlobal
+                     : (a->block_len <= kMaxLutWindow && a->key_bits == nullptr ? kLocal : kLocalWide);
     choose_runs(&p, mode, a->dtype, a->D);
     return finish(launch_fwd(p, a->dtype, a->D, mode, false, s), "t5a_fwd_sparse");
 }

@@ -481,6 +481,18 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     const T* qp = reinterpret_cast<const T*>(p.q) + q_off;
     T* op = reinterpret_cast<T*>(p.o) + o_off;
+    // local and block patterns, masks of any shape: validity of this sequence's tokens as a bit set (the global rows'
+    // key splits of the block pattern attend every key, as in the reference)
+    // (local pattern: the host sends such batches to the instantiation that masks per element, kLocalWide, so that
+    // the one with the window in the LUT carries none of this)
+    constexpr bool BITS = MODE == kLocalWide || MODE == kBlock;
+    const unsigned* kbits = (BITS && p.key_bits != nullptr && !gsplit) ? p.key_bits + (int64_t)b * p.key_bits_stride : nullptr;
+    // validity of the tokens pos0 .. pos0 + 63, bit e = token pos0 + e (wavefront-uniform: scalar loads)
+    auto token_bits = [&](int pos0) {
+        const int w = (pos0 + 32 * kKeyBitsFront) >> 5, sh = pos0 & 31;
+        const unsigned long long a = ((unsigned long long)kbits[w + 1] << 32) | kbits[w];
+        return sh != 0 ? (a >> sh) | ((unsigned long long)kbits[w + 2] << (64 - sh)) : a;
+    };
 
     // q tiles of this item: one, or a run of consecutive ones (RUNS)
     int qt_count = 1;
@@ -1037,6 +1049,17 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         d_tm = seg_end[0] / BN;                                // tiles from here on straddle the segment end
     }
     // sparse patterns: the class of a tile from the geometry of the current q tile (a few dozen scalar instructions)
+    // Validity of the 64 keys of a tile as the pattern's mask sees them (bit e = key j0 + e); kbits != nullptr.
+    auto tile_valid = [&](int sg, int j0) {
+        if (MODE != kBlock) return token_bits(j0);
+        // block pattern: list column c < block_len of [G global tokens | own block] takes the bit of token
+        // blk * block_len + c (the reference's mask layout, attentions.py:722-732)
+        if (sg == 0) return token_bits(blk * p.block_len + j0);            // global key j is column j
+        unsigned long long m = token_bits(j0 + p.aux);                      // own key j is column G + (j - blk * block_len)
+        const int e0 = (blk + 1) * p.block_len - p.aux - j0;                // tile position of the first column >= block_len:
+        if (e0 < 64) m |= ~0ull << max(e0, 0);                              // never masked (block 0: cut off by the segment's end)
+        return m;
+    };
     auto classify_sparse = [&](int t) {
         TileClass c;
         c.sg = 0; c.j0 = 0; c.side = 0; c.skip = true; c.use_lut = false; c.need_mask = false;
@@ -1066,6 +1089,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             int hole_lo, hole_span;
             block_hole(hole_lo, hole_span);
             c.need_mask = c.need_mask || (c.j0 < hole_lo + hole_span && c.j0 + BN > hole_lo);
+        }
+        if (BITS && kbits != nullptr && !c.skip) {
+            const unsigned long long m = tile_valid(c.sg, c.j0);
+            if (m == 0) c.skip = true;                 // no valid key in the tile
+            else if (m != ~0ull) c.need_mask = true;
         }
         c.side = (has_bias && !c.use_lut && !c.skip) ? (left_sat ? 1 : 2) : 0;
         if constexpr (win_lut) c.side = 0;
@@ -1259,6 +1287,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             if (MODE == kBlock && c.sg == 1) block_hole(hole_lo, hole_span);
             const unsigned hspan = (unsigned)hole_span;
             const int jh = c.j0 + 4 * hh - hole_lo;
+            // masks of any shape: this lane's keys of the tile's validity bits, bit `off` below
+            unsigned long long vm = ~0ull;
+            if (BITS && kbits != nullptr) vm = tile_valid(c.sg, c.j0) >> (4 * hh);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -1266,6 +1297,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     const int off = 32 * nt + 8 * (r >> 2) + (r & 3);
                     bool keep = (unsigned)(jl + off) < span;
                     if (MODE == kBlock) keep = keep && !((unsigned)(jh + off) < hspan);
+                    if (BITS) keep = keep && ((vm >> off) & 1ull) != 0;
                     st[nt][r] = keep ? st[nt][r] : -INFINITY;
                 }
         }
@@ -1460,6 +1492,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // q tiles whose tiles all have the same classes: away from the ends of the sequence (local pattern); whole
     // blocks other than the first, one q tile each, of a sequence without padding (block pattern)
     auto is_interior = [&]() {
+        if (BITS && kbits != nullptr) return false;   // (every q tile looks its keys' validity up)
         if (LOCAL) return seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
         if (MODE == kBlock) return !gsplit && tpb == 1 && blk >= 1 && (blk + 1) * p.block_len <= min(Nseq, n_valid) && i0 + BM <= Mseq;
         return false;

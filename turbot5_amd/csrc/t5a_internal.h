@@ -30,6 +30,7 @@ enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLoca
 // widest sliding window that is folded into the distance LUT (the LUT then spans 2 * (window + 96) distances;
 // 256 keeps it below 12 KB of LDS, so that two workgroups still share a compute unit)
 constexpr int kMaxLutWindow = 256;
+constexpr int kKeyBitsFront = 8;   // zero words in front of a sequence's validity bits (tiles start up to 255 keys early)
 
 struct FwdParams {
     const void* q; const void* k; const void* v; void* o; float* lse;
@@ -44,6 +45,9 @@ struct FwdParams {
     const int32_t* cu_q; const int32_t* cu_k;   // non-null: packed variable-length batch
     const int32_t* len_q; const int32_t* len_k; // optional lengths (rows between cu[b]+len[b] and cu[b+1] are padding)
     const int32_t* start_k;                     // sparse patterns, optional: first token of each sequence (left padding)
+    // local and block patterns, optional: token validity as a bit set, (B, key_bits_stride) words; token j is bit
+    // (j & 31) of word kKeyBitsFront + (j >> 5); zero words in front and behind
+    const uint32_t* key_bits; int64_t key_bits_stride;
     // packed batch with a launch plan (plan.hip): workgroup 8 k + x runs the item in plan[x][k]
     const int32_t* plan; const int32_t* plan_counts; int plan_slots;
     int B, H, M, N;

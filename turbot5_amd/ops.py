@@ -320,10 +320,40 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     return (o, lse) if return_lse else o
 
 
+KEY_BITS_FRONT = 8   # zero words in front of a sequence's validity bits (kKeyBitsFront of the library)
+
+
+def pack_key_bits(attention_mask: torch.Tensor, block_len: int, aux: int = 0) -> torch.Tensor:
+    """(B, L) mask (non-zero = token) -> (B, words) int32 bit sets as ``t5a_sparse_args.key_bits`` wants them: token j
+    is bit (j & 31) of word 8 + (j >> 5), zero words in front and behind.  Runs on the mask's device, no host sync."""
+    if attention_mask.dim() != 2:
+        raise ValueError("attention_mask must be (B, L)")
+    B, Lm = attention_mask.shape
+    words = int(L.load().t5a_sparse_key_bits_words(Lm, int(block_len), int(aux)))
+    body = (Lm + 31) // 32
+    valid = (attention_mask != 0)
+    if body * 32 != Lm:
+        valid = torch.nn.functional.pad(valid, (0, body * 32 - Lm))
+    weights = (torch.ones(32, dtype=torch.int64, device=valid.device) << torch.arange(32, device=valid.device))
+    packed = (valid.view(B, body, 32).to(torch.int64) * weights).sum(-1)            # 0 .. 2^32 - 1
+    packed = torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed).to(torch.int32)
+    out = torch.zeros(B, words, dtype=torch.int32, device=valid.device)
+    out[:, KEY_BITS_FRONT:KEY_BITS_FRONT + body] = packed
+    return out
+
+
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
-            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None, seq_starts=None):
+            NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None, seq_starts=None,
+            key_bits=None):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
+    if key_bits is not None:
+        if pattern == L.PATTERN_TGLOBAL or seq_lens is not None:
+            raise ValueError("key_bits is for the local and block patterns, instead of seq_lens")
+        need = int(L.load().t5a_sparse_key_bits_words(Lq, int(block_len), int(aux)))
+        if (key_bits.dtype != torch.int32 or key_bits.dim() != 2 or key_bits.shape[0] != B or key_bits.shape[1] < need
+                or key_bits.device != q.device or not key_bits.is_contiguous()):
+            raise ValueError(f"key_bits must be a contiguous int32 tensor (B, >= {need}) on the device of q: pack_key_bits()")
     for name, t in (("seq_lens", seq_lens), ("seq_starts", seq_starts)):
         if t is not None and (t.dtype != torch.int32 or t.shape != (B,) or t.device != q.device or not t.is_contiguous()):
             raise ValueError(f"{name} must be a contiguous int32 tensor of shape (B,) on the device of q")
@@ -355,8 +385,10 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
         a.seq_lens = seq_lens.data_ptr()
     if seq_starts is not None:
         a.seq_starts = seq_starts.data_ptr()
+    if key_bits is not None:
+        a.key_bits, a.key_bits_stride = key_bits.data_ptr(), key_bits.shape[1]
     # the local pattern's work items fetch LUT images that have the window folded in (windows up to 256)
-    window = int(block_len) if pattern == L.PATTERN_LOCAL and int(block_len) <= 256 else 0
+    window = int(block_len) if pattern == L.PATTERN_LOCAL and int(block_len) <= 256 and key_bits is None else 0
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, window=window)
     lib = L.load()
     ws_bytes = lib.t5a_sparse_workspace_bytes(pattern, B, H, Lq, D, int(block_len), int(aux))
@@ -371,29 +403,31 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
 
 
 def local_attention_with_fusing_bias(q, k, v, bias, block_len, sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                     seq_lens=None, exact_scores=None, seq_starts=None):
+                                     seq_lens=None, exact_scores=None, seq_starts=None, key_bits=None):
     """Sliding-window self-attention: key j visible to query i iff |j-i| < block_len, bias bucket(j-i).
 
     The op of T5LocalAttention (src/turbot5/model/attentions.py:583-638) without
     blocking, K/V triplication or a bias tensor.  q,k,v (B,H,L,D).
     ``seq_lens`` / ``seq_starts`` (B,) int32: the tokens of sequence b are the rows [start, start + len) (start
     defaults to 0: right padding); keys outside them are not attended (the mask of
-    src/turbot5/model/utils.py:174-188 for the sequence's own rows), positions stay the row indices."""
+    src/turbot5/model/utils.py:174-188 for the sequence's own rows), positions stay the row indices.
+    ``key_bits`` (``pack_key_bits(mask, block_len)``, instead of seq_lens): the same for a mask of any shape."""
     return _sparse(L.PATTERN_LOCAL, q, k, v, bias, block_len, 0, None, None, sm_scale, NUM_BUCKETS, MAX_DISTANCE,
-                   seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts)
+                   seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts, key_bits=key_bits)
 
 
 def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scale=1.0, NUM_BUCKETS=32,
-                                     MAX_DISTANCE=128, key_splits=True, exact_scores=None, seq_lens=None):
+                                     MAX_DISTANCE=128, key_splits=True, exact_scores=None, seq_lens=None, key_bits=None):
     """Block attention with ``n_global`` leading global tokens, the op of T5BlockAttention
     (src/turbot5/model/attentions.py:788-853) with the reference's key/mask layout.
 
     ``key_splits``: hand the library a workspace so that the global rows (which attend every key) are
     spread over the device as key splits and merged; False keeps them in one workgroup per (batch, head).
     ``seq_lens`` (B,) int32: valid tokens of each right-padded sequence, masked the way the reference lays its
-    padding mask over the key list (attentions.py:722-732); the global rows see every key regardless (:788-800)."""
+    padding mask over the key list (attentions.py:722-732); the global rows see every key regardless (:788-800).
+    ``key_bits`` (``pack_key_bits(mask, block_len, n_global)``): the same for a mask of any shape."""
     return _sparse(L.PATTERN_BLOCK, q, k, v, bias, block_len, n_global, None, None, sm_scale, NUM_BUCKETS,
-                   MAX_DISTANCE, key_splits=key_splits, exact_scores=exact_scores, seq_lens=seq_lens)
+                   MAX_DISTANCE, key_splits=key_splits, exact_scores=exact_scores, seq_lens=seq_lens, key_bits=key_bits)
 
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
