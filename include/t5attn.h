@@ -101,7 +101,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 111
+#define T5A_ABI_VERSION 112
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -207,7 +207,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *           [G global tokens | own block] is masked iff token b * block_len + c is padding, the last G
  *           columns never (always in block 0); the first G rows attend every key, padding included
  *           (:788-800).
- * key_bits (optional, LOCAL and BLOCK; instead of seq_lens / seq_starts): validity of every token as a bit set,
+ * key_bits (optional; instead of seq_lens / seq_starts): validity of every token as a bit set,
  * for attention masks of any shape (holes, padding on either side).  (B, key_bits_stride) uint32 words on the
  * device; token j of sequence b is bit (j & 31) of word 8 + (j >> 5) -- eight zero words in front, and zero words
  * behind the last token up to at least t5a_sparse_key_bits_words(L, block_len, aux) words in all.
@@ -216,6 +216,10 @@ int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
  *   BLOCK   the reference's additive mask as it lays it out (attentions.py:722-732), for any mask: list column
  *           c < block_len of [G global tokens | own block] is masked iff token b * block_len + c has bit 0, the
  *           last G columns never (always in block 0); the first G rows attend every key.
+ *   TGLOBAL window keys whose bit is 0 are not attended.  side_counts[b] = number of aux-block END positions
+ *           (rows p with p % aux == aux - 1) of sequence b whose bit is 1: it has that many side tokens, a
+ *           token's side token being min(row / aux, count - 1) (the reference's block ids for any mask,
+ *           src/turbot5/model/utils.py:191-237).
  * workspace (optional, BLOCK only): t5a_sparse_workspace_bytes() bytes of device memory.  With it
  * the G global rows, which attend all L keys, are computed as key splits spread over the whole
  * device and merged; without it they run as one workgroup per (batch, head).  Results agree to
@@ -235,6 +239,7 @@ typedef struct t5a_sparse_args {
     const int32_t* seq_starts;
     const uint32_t* key_bits;
     int64_t key_bits_stride;      /* words per sequence */
+    const int32_t* side_counts;   /* TGLOBAL with key_bits: (B) int32, side tokens of each sequence */
 } t5a_sparse_args;
 /* words per sequence that key_bits needs (front padding, ceil(L / 32), back padding) */
 int64_t t5a_sparse_key_bits_words(int32_t L, int32_t block_len, int32_t aux);
@@ -316,6 +321,11 @@ typedef struct t5a_rmsnorm_args {
     const void* residual; void* sum_out; int64_t residual_row_stride;
     const int32_t* seq_lens;
     const int32_t* seq_starts;   /* optional, with seq_lens: first valid row of each batch element (NULL = 0) */
+    /* optional (group > 1, instead of seq_lens): token validity bit sets laid out as for the sparse patterns; any
+     * stride that covers the rows will do: the buffer made for the attention call serves; and the number of groups of each batch element (the END positions of groups
+     * whose bit is 1): group g sums the valid rows of [g * group, (g + 1) * group), the last group every valid
+     * row from its start on; rows past the groups are zero. */
+    const uint32_t* key_bits; int64_t key_bits_stride; const int32_t* group_counts;
 } t5a_rmsnorm_args;
 int t5a_rmsnorm(const t5a_rmsnorm_args* args, t5a_stream_t stream);
 

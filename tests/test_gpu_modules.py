@@ -68,12 +68,10 @@ def test_attention_module_output_tuple(gpu_device):
         for name in ("local", "block", "transient-global"):
             out = T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device).eval()(x, mask=mask)
             assert torch.isfinite(out[0][mask.bool()]).all()
-        mask[1, 20:30] = 0                           # holes: local and block (validity bit sets)
-        for name in ("local", "block"):
+        mask[1, 20:30] = 0                           # holes: validity bit sets
+        for name in ("local", "block", "transient-global"):
             out = T5ATTENTION_TYPES[name](cfg, has_relative_attention_bias=True).to(gpu_device).eval()(x, mask=mask)
             assert torch.isfinite(out[0][mask.bool()]).all()
-    with pytest.raises(NotImplementedError):
-        T5ATTENTION_TYPES["transient-global"](cfg, has_relative_attention_bias=True).to(gpu_device)(x, mask=mask)
 
 
 def test_flash_encoder_with_padding(gpu_device):
@@ -337,6 +335,19 @@ def test_transient_global_encoder_with_right_padding(gpu_device):
     with torch.no_grad():
         got = m(ids.to(gpu_device), left.to(gpu_device)).cpu()
     assert (got[left.bool()] - want[left.bool()]).abs().max().item() <= 2e-3
+    # masks with holes: validity bit sets and a side-token count per sequence -- a side block whose END token is
+    # masked (its tokens still have their side token while a later END is valid), a masked tail, scattered holes
+    holes = torch.ones(3, 256)
+    holes[0, 40:50] = 0              # covers the END of side block 5 (row 47)
+    holes[0, 250:] = 0
+    holes[1, ::7] = 0
+    holes[1, :20] = 0
+    holes[2, 100:180] = 0
+    holes[2, 255] = 0                # the last END: rows 248..254 join side token 30
+    want = OM.encoder_forward(sd, cfg, ids, holes, attention_type="transient-global")
+    with torch.no_grad():
+        got = m(ids.to(gpu_device), holes.to(gpu_device)).cpu()
+    assert (got[holes.bool()] - want[holes.bool()]).abs().max().item() <= 2e-3
 
 
 def test_block_encoder_with_right_padding(gpu_device):

@@ -151,3 +151,34 @@ def test_side_token_producer_with_sequence_lengths(gpu_device, dtype, L, gbs, le
     assert (one.float().cpu() - want1.float()).abs().max().item() <= tol * max(1.0, want1.float().abs().max().item())
     with pytest.raises(ValueError):
         rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=1, seq_lens=tl, residual=hidden.to(gpu_device))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("L,gbs", [(512, 16), (100, 16), (64, 8), (777, 32)])
+def test_side_token_producer_with_masks_of_any_shape(gpu_device, dtype, L, gbs):
+    """key_bits and group_counts: a side token sums the valid tokens of its block, the last one every valid token
+    from its block on, rows past the count are zero -- the oracle's block ids and aggregates for any mask"""
+    from turbot5_amd.ops import pack_key_bits, rms_norm, side_token_counts
+    B, d = 5, 256
+    g = torch.Generator().manual_seed(L * 7 + gbs)
+    hidden = torch.randn(B, L, d, generator=g).to(DT[dtype])
+    w = (1.0 + 0.1 * torch.randn(d, generator=g)).to(DT[dtype])
+    mask = torch.ones(B, L)
+    mask[0] = (torch.rand(L, generator=g) > 0.3).float()
+    mask[1, : L // 3] = 0
+    mask[2, L // 5: L // 2] = 0
+    mask[2, -(gbs + 3):] = 0
+    mask[3, gbs - 1::gbs] = 0          # no block END is valid: no side token
+    want = tglobal_side_inputs(hidden, gbs, w, 1e-6, mask)
+    dmask = mask.to(gpu_device)
+    counts = side_token_counts(dmask, gbs)
+    got = rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=gbs, key_bits=pack_key_bits(dmask, gbs),
+                   group_counts=counts)
+    assert got.shape == want.shape == (B, L // gbs, d)
+    tol = 1e-5 if dtype == "f32" else 2e-2
+    assert (got.float().cpu() - want.float()).abs().max().item() <= tol * max(1.0, want.float().abs().max().item())
+    assert (got[3] == 0).all() and counts[3].item() == 0
+    for b in range(B):
+        assert (got[b, counts[b].item():] == 0).all()
+    with pytest.raises(ValueError):
+        rms_norm(hidden.to(gpu_device), w.to(gpu_device), 1e-6, group=gbs, key_bits=pack_key_bits(dmask, gbs))

@@ -428,3 +428,30 @@ def test_block_with_masks_of_any_shape(gpu_device, dtype, L, Bl, G):
     rows = mask.bool()[:, None, :, None].expand_as(out) & torch.isfinite(out)
     assert (out - want)[rows].abs().max().item() <= TOL[dtype]
     assert rows.float().mean().item() > 0.5
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("L,Bl,gbs", [(512, 128, 16), (384, 64, 8), (640, 32, 16), (1000, 127, 16), (300, 64, 32)])
+def test_tglobal_with_masks_of_any_shape(gpu_device, dtype, L, Bl, gbs):
+    """key_bits and side_counts: window keys by their validity, side tokens counted by the valid block ENDs, a
+    token's side token min(row // gbs, count - 1) (utils.py:191-237); rows of valid tokens against the oracle"""
+    from turbot5_amd import ops
+    B, H, D = 5, 2, 64
+    q, k, v = (rnd(B, H, L, D, seed=180 + i, dtype=dtype) for i in range(3))
+    sk, sv = (rnd(B, H, L // gbs, D, seed=183 + i, dtype=dtype) for i in range(2))
+    table = rnd(32, H, seed=185, scale=1.0)
+    mask = _random_masks(B, L, 186)
+    dmask = mask.to(gpu_device)
+    bits = ops.pack_key_bits(dmask, Bl, gbs)
+    counts = ops.side_token_counts(dmask, gbs)
+    assert counts.tolist() == [int(mask[b, gbs - 1::gbs].sum()) for b in range(B)]
+    out = ops.transient_global_attention_with_fusing_bias(
+        *(t.to(gpu_device) for t in (q, k, v, sk, sv)), table.to(gpu_device), Bl, gbs, key_bits=bits,
+        side_counts=counts).float().cpu()
+    want = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, gbs, mask)
+    rows = mask.bool()[:, None, :, None].expand_as(out)
+    assert torch.isfinite(out[rows]).all()
+    assert (out - want)[rows].abs().max().item() <= TOL[dtype]
+    with pytest.raises(ValueError):   # the counts are not optional
+        ops.transient_global_attention_with_fusing_bias(
+            *(t.to(gpu_device) for t in (q, k, v, sk, sv)), table.to(gpu_device), Bl, gbs, key_bits=bits)

@@ -35,9 +35,38 @@ def test_struct_sizes_follow_the_header(lib):
     assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8 + 2 * 4
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
-    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 4 * 8
+    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 5 * 8
     assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4 + 2 * 8
-    assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 5 * 8
+    assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 5 * 8 + 3 * 8
+
+
+def test_key_bits_layout_and_size(lib):
+    """Token j is bit (j & 31) of word 8 + (j >> 5); zero words in front and behind, as many as the kernels' tiles
+    may look at; the side-token count is the number of valid block ENDs."""
+    from turbot5_amd import ops
+    handle = lib.load()
+    assert handle.t5a_sparse_key_bits_words(1000, 128, 16) == 8 + (1000 + 256 + 16 + 256 + 31) // 32 + 4
+    assert handle.t5a_sparse_key_bits_words(-1, 128, 0) == -1 and handle.t5a_sparse_key_bits_words(10, 0, 0) == -1
+    g = torch.Generator().manual_seed(5)
+    for Lm in (1, 31, 32, 33, 100, 257):
+        mask = (torch.rand(3, Lm, generator=g) > 0.4).float()
+        mask[2] = 1
+        bits = ops.pack_key_bits(mask, 64, 8)
+        assert bits.dtype == torch.int32 and bits.shape == (3, handle.t5a_sparse_key_bits_words(Lm, 64, 8))
+        words = bits.to(torch.int64) & 0xFFFFFFFF
+        for b in range(3):
+            for j in range(Lm):
+                assert (int(words[b, ops.KEY_BITS_FRONT + (j >> 5)]) >> (j & 31)) & 1 == int(mask[b, j]), (Lm, b, j)
+        assert (words[:, :ops.KEY_BITS_FRONT] == 0).all()
+        tail = words[:, ops.KEY_BITS_FRONT + (Lm + 31) // 32:]
+        assert (tail == 0).all()
+        if Lm % 32:   # bits past the last token stay zero
+            assert (int(words[2, ops.KEY_BITS_FRONT + Lm // 32]) >> (Lm % 32)) == 0
+    mask = torch.ones(2, 50)
+    mask[0, 15] = 0
+    mask[1, 40:] = 0
+    assert ops.side_token_counts(mask, 16).tolist() == [2, 2]
+    assert ops.side_token_counts(mask, 8).tolist() == [5, 5]
 
 
 @pytest.mark.parametrize("bidirectional", [True, False])

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 111   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 112   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
@@ -67,7 +67,7 @@ class T5ASparseArgs(C.Structure):
                 ("pattern", C.c_int32), ("block_len", C.c_int32), ("aux", C.c_int32), ("n_side", C.c_int32),
                 ("sm_scale", C.c_float), ("exact_scores", C.c_int32),
                 ("bias", T5ABias), ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p),
-                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64)]
+                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64), ("side_counts", C.c_void_p)]
 
 
 class T5ASplitKArgs(C.Structure):
@@ -87,7 +87,8 @@ class T5ARmsNormArgs(C.Structure):
                 ("x_dtype", C.c_int32), ("weight_dtype", C.c_int32), ("eps", C.c_float),
                 ("reserved", C.c_int32),
                 ("residual", C.c_void_p), ("sum_out", C.c_void_p), ("residual_row_stride", C.c_int64),
-                ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p)]
+                ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p),
+                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64), ("group_counts", C.c_void_p)]
 
 
 _lib = None

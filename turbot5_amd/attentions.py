@@ -43,13 +43,15 @@ class T5LayerNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(dim))
 
     def forward(self, x: torch.Tensor, group: int = 1, seq_lens: Optional[torch.Tensor] = None,
-                seq_starts: Optional[torch.Tensor] = None) -> torch.Tensor:
+                seq_starts: Optional[torch.Tensor] = None, key_bits: Optional[torch.Tensor] = None,
+                group_counts: Optional[torch.Tensor] = None) -> torch.Tensor:
         """On a ROCm device: the fused HIP kernel (the reference switches to its Triton kernel there,
         modules.py:61-66).  Host tensors take the reference's eager formula (modules.py:51-59).
         ``group`` > 1 norms the sums of ``group`` consecutive rows of each sequence (side tokens)."""
         if x.is_cuda:
             from .ops import rms_norm
-            return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens, seq_starts=seq_starts)
+            return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens, seq_starts=seq_starts,
+                            key_bits=key_bits, group_counts=group_counts)
         if group > 1:
             B, L, d = x.shape
             n = L // group
@@ -362,12 +364,11 @@ class _SparseBase(_T5AttentionBase):
             bits = plans[key] = ops.pack_key_bits(mask, block_len, aux)
         return bits
 
-    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions, left_padding_ok=True,
-                    bits_ok=False):
+    def _check_call(self, mask, layer_head_mask, past_key_value, use_cache, output_attentions, left_padding_ok=True):
         """-> (lengths, first rows): (B,) int32 device tensors for a batch whose rows are each ONE run of valid
         tokens (padding on the right, and on the left where the pattern takes it); (None, None) for all ones.
-        First rows are None for right padding.  ``bits_ok``: any other mask gives ("bits", None) -- the caller passes
-        validity bit sets instead."""
+        First rows are None for right padding.  Any other mask gives ("bits", None): the caller passes validity
+        bit sets instead."""
         if past_key_value is not None:
             warnings.warn('Currently, passing past key value states is not supported.')
         if use_cache is not None:
@@ -387,12 +388,7 @@ class _SparseBase(_T5AttentionBase):
                             starts = plans["starts"] = (unpad[1][1][:B] - torch.arange(
                                 B, device=mask.device, dtype=torch.int32) * L).contiguous()
                         return unpad[1][0], starts
-                if bits_ok:
-                    return "bits", None
-                raise NotImplementedError(
-                    f"{type(self).__name__} runs as tile skipping for attention masks whose rows are one run of valid "
-                    "tokens (padding on the right" + (" or on the left" if left_padding_ok else "")
-                    + "); use attention_type='flash' for masks with holes")
+                return "bits", None
         return None, None
 
     def _qkv(self, hidden_states):
@@ -417,8 +413,7 @@ class T5LocalAttention(_SparseBase):
                 use_cache=None, output_attentions=False):
         # right-padded batches: the keys of a sequence end at its length (the key half of the reference's
         # local mask, utils.py:174-188); outputs at padded positions mean nothing, as in the reference
-        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                                                bits_ok=True)
+        seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
         q, k, v = self._qkv(hidden_states)
         table = self._table(position_bias)
         # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
@@ -446,7 +441,7 @@ class T5BlockAttention(_SparseBase):
         # right-padded batches: the reference's additive mask over its key list (attentions.py:722-732)
         # (left padding and holes: validity bit sets, looked up per tile)
         seq_lens, _ = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
-                                       left_padding_ok=False, bits_ok=True)
+                                       left_padding_ok=False)
         if seq_lens is not None and hidden_states.shape[1] < self.block_len:
             raise NotImplementedError("T5BlockAttention: padded batches shorter than one block are not supported")
         q, k, v = self._qkv(hidden_states)
@@ -474,17 +469,19 @@ class T5TransientGlobalAttention(_SparseBase):
         self.global_input_layer_norm = T5LayerNorm(config.d_model, eps=config.layer_norm_epsilon)
 
     def side_inputs(self, hidden_states: torch.Tensor, seq_lens: Optional[torch.Tensor] = None,
-                    seq_starts: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    seq_starts: Optional[torch.Tensor] = None, key_bits: Optional[torch.Tensor] = None,
+                    side_counts: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Normalised block sums, (B, L // global_block_size, d_model); trailing tokens that do not fill
         a block join the last one (utils.py:206-212, :249-258; attentions.py:959-966).  With ``seq_lens``
-        each right-padded sequence counts its valid tokens only."""
+        (or ``key_bits`` and ``side_counts``, for masks of any shape) each sequence counts its valid tokens only."""
         B, L, d = hidden_states.shape
         gbs = self.global_block_size
         n_side = L // gbs
         if n_side == 0:
             return hidden_states.new_zeros(B, 0, d)
         # block sums and norm in one kernel
-        return self.global_input_layer_norm(hidden_states, group=gbs, seq_lens=seq_lens, seq_starts=seq_starts)
+        return self.global_input_layer_norm(hidden_states, group=gbs, seq_lens=seq_lens, seq_starts=seq_starts,
+                                            key_bits=key_bits, group_counts=side_counts)
 
     def forward(self, hidden_states, mask=None, position_bias=None, layer_head_mask=None, past_key_value=None,
                 use_cache=None, output_attentions=False):
@@ -492,16 +489,24 @@ class T5TransientGlobalAttention(_SparseBase):
         seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
         batch_size = hidden_states.shape[0]
         adt = self._attn_dtype(hidden_states)
+        block_len = min(self.block_len, hidden_states.shape[1])
+        key_bits = side_counts = None
+        if isinstance(seq_lens, str):   # a mask with holes: validity bit sets and the side tokens of each sequence
+            seq_lens = None
+            key_bits = self._key_bits(mask, block_len, self.global_block_size)
+            plans = _mask_info(mask)[1][2]
+            side_counts = plans.get(("side_counts", self.global_block_size))
+            if side_counts is None:
+                side_counts = plans[("side_counts", self.global_block_size)] = ops.side_token_counts(mask, self.global_block_size)
         q, k, v = self._qkv(hidden_states)
-        side = self.side_inputs(hidden_states, seq_lens, seq_starts)
+        side = self.side_inputs(hidden_states, seq_lens, seq_starts, key_bits, side_counts)
         side_k = self._shape(self.k(side), batch_size).to(adt)
         side_v = self._shape(self.v(side), batch_size).to(adt)
         table = self._table(position_bias)
-        block_len = min(self.block_len, hidden_states.shape[1])
         out = ops.transient_global_attention_with_fusing_bias(
             q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
             self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens,
-            seq_starts=seq_starts, exact_scores=self._exact)
+            seq_starts=seq_starts, exact_scores=self._exact, key_bits=key_bits, side_counts=side_counts)
         return self._finish(out, hidden_states, table)
 
 

@@ -515,7 +515,8 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     p.len_k = a->seq_lens;
     p.start_k = a->seq_starts;
     if (a->key_bits != nullptr) {
-        if (a->pattern == T5A_PATTERN_TGLOBAL) return fail(T5A_ERR_PATTERN, "key_bits is for the local and block patterns");
+        if (a->pattern == T5A_PATTERN_TGLOBAL && a->side_counts == nullptr)
+            return fail(T5A_ERR_NULL, "transient-global pattern: key_bits needs side_counts");
         if (a->seq_lens != nullptr) return fail(T5A_ERR_PATTERN, "key_bits and seq_lens are alternatives");
         const int64_t need = t5a_sparse_key_bits_words(a->L, a->block_len, a->aux);
         if (a->key_bits_stride < need)
@@ -526,6 +527,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
             return fail(T5A_ERR_PATTERN, "block pattern: key_bits with a sequence shorter than one block is not supported");
         p.key_bits = a->key_bits;
         p.key_bits_stride = a->key_bits_stride;
+        if (a->pattern == T5A_PATTERN_TGLOBAL) p.side_counts = a->side_counts;
     }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
     p.c1 = a->sm_scale * kLog2e;
@@ -615,7 +617,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     }
     p.tiles_per_seq = (a->L + 127) / 128;
     // (validity bit sets go with the instantiation that masks per element)
-    const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? kTGlobal
+    const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? (a->key_bits != nullptr ? kTGlobalBits : kTGlobal)
                      : (a->block_len <= kMaxLutWindow && a->key_bits == nullptr ? kLocal : kLocalWide);
     choose_runs(&p, mode, a->dtype, a->D);
     return finish(launch_fwd(p, a->dtype, a->D, mode, false, s), "t5a_fwd_sparse");
@@ -743,6 +745,16 @@ int t5a_rmsnorm(const t5a_rmsnorm_args* a, t5a_stream_t stream) {
         p.starts = a->seq_starts;
     } else if (a->seq_starts != nullptr) {
         return fail(T5A_ERR_SHAPE, "seq_starts needs seq_lens");
+    }
+    if (a->key_bits != nullptr) {
+        if (a->group <= 1 || a->seq_lens != nullptr || a->residual != nullptr)
+            return fail(T5A_ERR_SHAPE, "key_bits is for group > 1, without seq_lens or residual");
+        if (a->group_counts == nullptr) return fail(T5A_ERR_NULL, "key_bits needs group_counts");
+        const int64_t need = kKeyBitsFront + ((int64_t)a->rows_per_batch + 31) / 32;   // (only the rows' own bits are read)
+        if (a->key_bits_stride < need)
+            return fail(T5A_ERR_SHAPE, "key_bits_stride %lld, the rows need %lld words", (long long)a->key_bits_stride, (long long)need);
+        if ((reinterpret_cast<uintptr_t>(a->key_bits) & 3) != 0) return fail(T5A_ERR_STRIDE, "key_bits must be 4-byte aligned");
+        p.key_bits = a->key_bits; p.key_bits_stride = a->key_bits_stride; p.group_counts = a->group_counts;
     }
     p.x_batch_stride = a->x_strides[0]; p.x_row_stride = a->x_strides[1]; p.y_row_stride = a->dim;
     p.out_per_batch = out_per_batch;

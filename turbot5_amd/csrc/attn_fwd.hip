@@ -302,6 +302,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     constexpr int BN = G::BN, NT = G::NT;
     constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
     constexpr bool LOCAL = MODE == kLocal || MODE == kLocalWide;   // sliding window, one segment
+    constexpr bool TG = MODE == kTGlobal || MODE == kTGlobalBits;   // sliding window and side tokens
     // Sparse patterns, LDS-DMA geometries: a work item is a RUN of consecutive q tiles of one (batch, head).  Their
     // key tiles form one stream through the LDS rings (the requests for the next q tile's first tiles go out during
     // the last steps of the current one) and the distance LUT is built once per run; a q tile of a sparse pattern
@@ -457,14 +458,16 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         // windowed patterns on a right-padded batch: the keys of a sequence end at its length; positions are
         // the row indices, so nothing else changes (rows past the length see what is left of their window).
         // Its side tokens are the full blocks of that length, the rest of its tokens joining the last one.
-        if ((LOCAL || MODE == kTGlobal) && p.len_k != nullptr) {
+        if ((LOCAL || TG) && p.len_k != nullptr) {
             // the sequence's tokens are the rows [key_lo, Nseq); a token's position stays its row index
             key_lo = p.start_k != nullptr ? max(0, min(p.N, p.start_k[b])) : 0;
             Nseq = max(key_lo, min(p.N, key_lo + max(0, p.len_k[b])));
             // side tokens: one per block END among the tokens; a token's side token is min(row / aux, count - 1)
             // (what the reference's block ids come to for one run of tokens, src/turbot5/model/utils.py:191-237)
-            if (MODE == kTGlobal) n_side = min(p.n_side, Nseq / p.aux - key_lo / p.aux);
+            if (TG) n_side = min(p.n_side, Nseq / p.aux - key_lo / p.aux);
         }
+        // masks of any shape: the caller counts the block ENDs among the valid tokens
+        if (TG && p.side_counts != nullptr) n_side = max(0, min(p.n_side, p.side_counts[b]));
         if (MODE == kBlock && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
@@ -481,11 +484,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     }
     const T* qp = reinterpret_cast<const T*>(p.q) + q_off;
     T* op = reinterpret_cast<T*>(p.o) + o_off;
-    // local and block patterns, masks of any shape: validity of this sequence's tokens as a bit set (the global rows'
+    // sparse patterns, masks of any shape: validity of this sequence's tokens as a bit set (the global rows'
     // key splits of the block pattern attend every key, as in the reference)
-    // (local pattern: the host sends such batches to the instantiation that masks per element, kLocalWide, so that
-    // the one with the window in the LUT carries none of this)
-    constexpr bool BITS = MODE == kLocalWide || MODE == kBlock;
+    // (local and transient-global patterns: the host sends such batches to instantiations of their own, kLocalWide
+    // and kTGlobalBits, so that the ones for batches without holes carry none of this)
+    constexpr bool BITS = MODE == kLocalWide || MODE == kBlock || MODE == kTGlobalBits;
     const unsigned* kbits = (BITS && p.key_bits != nullptr && !gsplit) ? p.key_bits + (int64_t)b * p.key_bits_stride : nullptr;
     // validity of the tokens pos0 .. pos0 + 63, bit e = token pos0 + e (wavefront-uniform: scalar loads)
     auto token_bits = [&](int pos0) {
@@ -522,9 +525,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     seg_start[0] = 0; seg_end[0] = 0;
     seg_start[1] = seg_end[1] = seg_lend[1] = 0; seg_kind[1] = 0; seg_win[1] = 0;
     seg_kind[0] = 0; seg_win[0] = 0; seg_lend[0] = Nseq;
-    if (LOCAL || MODE == kTGlobal) {
+    if (LOCAL || TG) {
         seg_win[0] = 1;
-        if (MODE == kTGlobal) {
+        if (TG) {
             nseg = 2;
             seg_k[1] = reinterpret_cast<const T*>(p.side_k) + (int64_t)b * p.sk_sb + (int64_t)h * p.sk_sh;
             seg_v[1] = reinterpret_cast<const T*>(p.side_v) + (int64_t)b * p.sv_sb + (int64_t)h * p.sv_sh;
@@ -570,7 +573,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
         if (DENSE) {
             seg_end[0] = CAUSAL ? max(0, min(Nseq, i0 + BM + P)) : Nseq;
-        } else if (LOCAL || MODE == kTGlobal) {
+        } else if (LOCAL || TG) {
             seg_start[0] = RUNS ? i0 - p.block_len + 1 : max(key_lo, i0 - p.block_len + 1);
             seg_end[0] = min(Nseq, min(i0 + BM, Mseq) - 1 + p.block_len);
         }
@@ -1051,6 +1054,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // sparse patterns: the class of a tile from the geometry of the current q tile (a few dozen scalar instructions)
     // Validity of the 64 keys of a tile as the pattern's mask sees them (bit e = key j0 + e); kbits != nullptr.
     auto tile_valid = [&](int sg, int j0) {
+        if (TG && sg == 1) return ~0ull;   // side tokens: the count of them is the mask
         if (MODE != kBlock) return token_bits(j0);
         // block pattern: list column c < block_len of [G global tokens | own block] takes the bit of token
         // blk * block_len + c (the reference's mask layout, attentions.py:722-732)
@@ -1068,7 +1072,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const int kind = (c.sg ? seg_kind[1] : seg_kind[0]);
         const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
         (void)kind;
-        constexpr bool cached = MODE == kBlock || MODE == kTGlobal;   // positions kept per q tile (set_positions)
+        constexpr bool cached = MODE == kBlock || TG;   // positions kept per q tile (set_positions)
         const int qlo = cached ? (c.sg ? wq_lo[1] : wq_lo[0]) : iw0 + P, qhi = cached ? (c.sg ? wq_hi[1] : wq_hi[0]) : iw1 + P;
         const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
         c.skip = iw0 >= row_end;                              // wavefront without live rows
@@ -1167,7 +1171,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (kind == 1) return row % p.block_len + p.aux;
         return min(row / p.aux, n_side - 1);   // trailing tokens past the last full block join it
     };
-    constexpr bool POS_CACHE = MODE == kBlock || MODE == kTGlobal;   // (the other patterns' positions are row + P)
+    constexpr bool POS_CACHE = MODE == kBlock || TG;   // (the other patterns' positions are row + P)
     auto set_positions = [&]() {
         if constexpr (!POS_CACHE) return;
         const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
@@ -1277,7 +1281,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0 && !win_lut;
             const int qpos = lane_qpos(c.sg);
             // this lane's row sees the keys [lo, hi): one subtraction and one unsigned compare per element
-            const int seg_lo = (c.sg == 0 && (LOCAL || MODE == kTGlobal)) ? key_lo : 0;   // first key of the sequence
+            const int seg_lo = (c.sg == 0 && (LOCAL || TG)) ? key_lo : 0;   // first key of the sequence
             const int lo = win ? max(seg_lo, qpos - p.block_len + 1) : seg_lo;
             const int hi = win ? min(s_end, qpos + p.block_len) : s_end;
             const unsigned span = (unsigned)max(hi - lo, 0);
@@ -1890,6 +1894,7 @@ static hipError_t launch_mode(const FwdParams& p, int mode, bool causal, hipStre
         case kLocalWide: return launch_one<T, D, kLocalWide, false>(p, s);
         case kBlock: return launch_one<T, D, kBlock, false>(p, s);
         case kTGlobal: return launch_one<T, D, kTGlobal, false>(p, s);
+        case kTGlobalBits: return launch_one<T, D, kTGlobalBits, false>(p, s);
     }
     return hipErrorInvalidValue;
 }

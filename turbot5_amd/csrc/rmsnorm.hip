@@ -49,11 +49,18 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     // among its rows, group g taking its rows of [g * group, (g + 1) * group) and the last group every row from
     // there on (the reference's block ids for one run of tokens: min(row / group, groups - 1),
     // src/turbot5/model/utils.py:191-237); groups without a row and output rows past the groups are zero.
-    const int start_b = p.starts ? max(0, min(p.rows_per_batch, p.starts[b])) : 0;
-    const int end_b = p.lens ? min(p.rows_per_batch, start_b + max(0, p.lens[b])) : p.rows_per_batch;
-    const int groups_b = p.lens ? end_b / p.group - start_b / p.group : p.out_per_batch;
+    // With validity bit sets (masks of any shape) the groups are counted by the caller and a group sums its valid rows.
+    const unsigned* kbits = p.key_bits != nullptr ? p.key_bits + b * p.key_bits_stride : nullptr;
+    const int start_b = (p.starts && !kbits) ? max(0, min(p.rows_per_batch, p.starts[b])) : 0;
+    const int end_b = (p.lens && !kbits) ? min(p.rows_per_batch, start_b + max(0, p.lens[b])) : p.rows_per_batch;
+    const int groups_b = kbits ? max(0, min(p.out_per_batch, p.group_counts[b]))
+                               : (p.lens ? end_b / p.group - start_b / p.group : p.out_per_batch);
     const int first = max(start_b, g * p.group);
     const int count = (g == groups_b - 1 ? end_b : min((g + 1) * p.group, end_b)) - first;
+    auto row_valid = [&](int r) {   // token first + r of this batch element (wavefront-uniform)
+        const int tok = first + r;
+        return ((kbits[kKeyBitsFront + (tok >> 5)] >> (tok & 31)) & 1u) != 0;
+    };
     const TX* x = reinterpret_cast<const TX*>(p.x) + b * p.x_batch_stride + (int64_t)first * p.x_row_stride;
     const TX* res = p.residual ? reinterpret_cast<const TX*>(p.residual) + row * p.residual_row_stride : nullptr;
     TX* sum = res ? reinterpret_cast<TX*>(p.sum_out) + row * p.y_row_stride : nullptr;
@@ -71,6 +78,19 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsParams p) {
     // chunk c of the row to normalise, as the input type holds it: the input row, or the sum of `count`
     // rows, or input + residual -- each sum rounded to the input type, as the torch expression leaves it
     auto load = [&](int c, float (&f)[VEC]) {
+        if (kbits != nullptr) {   // the sum of the group's valid rows
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) f[i] = 0.f;
+            for (int r = 0; r < count; ++r) {
+                if (!row_valid(r)) continue;
+                const Vec<TX, VEC> u = *reinterpret_cast<const Vec<TX, VEC>*>(x + (int64_t)r * p.x_row_stride + c * VEC);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) f[i] += Cvt<TX>::up(u.v[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) f[i] = Cvt<TX>::up(Cvt<TX>::down(f[i]));
+            return;
+        }
         const Vec<TX, VEC> v = *reinterpret_cast<const Vec<TX, VEC>*>(x + c * VEC);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) f[i] = Cvt<TX>::up(v.v[i]);

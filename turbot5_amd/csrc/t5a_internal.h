@@ -25,8 +25,8 @@ struct BucketSpec {
 // kPacked: dense semantics per sequence of a packed batch (cu_seqlens); a separate instantiation, so that
 // the unpacked kernel carries none of its work-item search
 // kLocal: sliding window of at most kMaxLutWindow, folded into the distance LUT; kLocalWide: wider windows, masked
-// per element at their edges
-enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLocalWide = 5 };
+// per element at their edges, and masks of any shape; kTGlobalBits: transient-global with masks of any shape
+enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLocalWide = 5, kTGlobalBits = 6 };
 // widest sliding window that is folded into the distance LUT (the LUT then spans 2 * (window + 96) distances;
 // 256 keeps it below 12 KB of LDS, so that two workgroups still share a compute unit)
 constexpr int kMaxLutWindow = 256;
@@ -48,6 +48,7 @@ struct FwdParams {
     // local and block patterns, optional: token validity as a bit set, (B, key_bits_stride) words; token j is bit
     // (j & 31) of word kKeyBitsFront + (j >> 5); zero words in front and behind
     const uint32_t* key_bits; int64_t key_bits_stride;
+    const int32_t* side_counts;                 // transient-global pattern with key_bits: side tokens per sequence
     // packed batch with a launch plan (plan.hip): workgroup 8 k + x runs the item in plan[x][k]
     const int32_t* plan; const int32_t* plan_counts; int plan_slots;
     int B, H, M, N;
@@ -127,6 +128,8 @@ struct RmsParams {
     const void* residual; void* sum_out;                  // optional: normalise x + residual, write the sum (input type)
     const int* lens;                                      // optional (group > 1): valid rows per batch element
     const int* starts;                                    // optional, with lens: first valid row per batch element
+    const uint32_t* key_bits; int64_t key_bits_stride;    // optional (group > 1): token validity bit sets ...
+    const int* group_counts;                              // ... and the groups per batch element
     int64_t residual_row_stride;
     int64_t x_batch_stride, x_row_stride, y_row_stride;   // elements
     int64_t out_rows;        // batches * out_per_batch

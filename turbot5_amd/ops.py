@@ -342,14 +342,26 @@ def pack_key_bits(attention_mask: torch.Tensor, block_len: int, aux: int = 0) ->
     return out
 
 
+def side_token_counts(attention_mask: torch.Tensor, global_block_size: int) -> torch.Tensor:
+    """(B, L) mask -> (B,) int32: the side tokens of each sequence, one per valid token at the END of a block of
+    ``global_block_size`` positions (src/turbot5/model/utils.py:206-216).  On the mask's device, no host sync."""
+    g = int(global_block_size)
+    return (attention_mask[:, g - 1::g] != 0).sum(-1).to(torch.int32).contiguous()
+
+
 def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm_scale=1.0,
             NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None, seq_starts=None,
-            key_bits=None):
+            key_bits=None, side_counts=None):
     _check_inputs(q, k, v)
     B, H, Lq, D = q.shape
+    if side_counts is not None and (pattern != L.PATTERN_TGLOBAL or key_bits is None):
+        raise ValueError("side_counts goes with key_bits in the transient-global pattern")
     if key_bits is not None:
-        if pattern == L.PATTERN_TGLOBAL or seq_lens is not None:
-            raise ValueError("key_bits is for the local and block patterns, instead of seq_lens")
+        if seq_lens is not None:
+            raise ValueError("key_bits is instead of seq_lens")
+        if pattern == L.PATTERN_TGLOBAL and (side_counts is None or side_counts.dtype != torch.int32 or side_counts.shape != (B,)
+                                             or side_counts.device != q.device or not side_counts.is_contiguous()):
+            raise ValueError("transient-global attention with key_bits needs side_counts: side_token_counts(mask, global_block_size)")
         need = int(L.load().t5a_sparse_key_bits_words(Lq, int(block_len), int(aux)))
         if (key_bits.dtype != torch.int32 or key_bits.dim() != 2 or key_bits.shape[0] != B or key_bits.shape[1] < need
                 or key_bits.device != q.device or not key_bits.is_contiguous()):
@@ -387,6 +399,8 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
         a.seq_starts = seq_starts.data_ptr()
     if key_bits is not None:
         a.key_bits, a.key_bits_stride = key_bits.data_ptr(), key_bits.shape[1]
+        if side_counts is not None:
+            a.side_counts = side_counts.data_ptr()
     # the local pattern's work items fetch LUT images that have the window folded in (windows up to 256)
     window = int(block_len) if pattern == L.PATTERN_LOCAL and int(block_len) <= 256 and key_bits is None else 0
     a.bias, keep = _bias_struct(bias, H, NUM_BUCKETS, MAX_DISTANCE, q, window=window)
@@ -432,19 +446,23 @@ def block_attention_with_fusing_bias(q, k, v, bias, block_len, n_global, sm_scal
 
 def transient_global_attention_with_fusing_bias(q, k, v, side_k, side_v, bias, block_len, global_block_size,
                                                 sm_scale=1.0, NUM_BUCKETS=32, MAX_DISTANCE=128, seq_lens=None,
-                                                exact_scores=None, seq_starts=None):
+                                                exact_scores=None, seq_starts=None, key_bits=None, side_counts=None):
     """Sliding window plus side tokens, the op of T5TransientGlobalAttention
     (src/turbot5/model/attentions.py:977-1052).  side_k/side_v (B,H,L//global_block_size,D).
     ``seq_lens`` / ``seq_starts`` (B,) int32: the tokens of sequence b are the rows [start, start + len); it has
     (start + len) // global_block_size - start // global_block_size side tokens
-    (src/turbot5/model/utils.py:191-237 for one run of tokens) and only its own rows as keys."""
+    (src/turbot5/model/utils.py:191-237 for one run of tokens) and only its own rows as keys.
+    ``key_bits`` (``pack_key_bits(mask, block_len, global_block_size)``) with ``side_counts``
+    (``side_token_counts(mask, global_block_size)``), instead of seq_lens: the same for a mask of any shape."""
     return _sparse(L.PATTERN_TGLOBAL, q, k, v, bias, block_len, global_block_size, side_k, side_v, sm_scale,
-                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts)
+                   NUM_BUCKETS, MAX_DISTANCE, seq_lens=seq_lens, exact_scores=exact_scores, seq_starts=seq_starts,
+                   key_bits=key_bits, side_counts=side_counts)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: int = 1,
              residual: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None,
-             seq_starts: Optional[torch.Tensor] = None):
+             seq_starts: Optional[torch.Tensor] = None, key_bits: Optional[torch.Tensor] = None,
+             group_counts: Optional[torch.Tensor] = None):
     """T5 RMS norm over the last dimension (src/turbot5/model/modules.py:51-59).
 
     With ``residual`` (same shape and dtype as x, group 1) the kernel normalises ``x + residual`` and
@@ -457,6 +475,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
     ``seq_lens`` / ``seq_starts`` (B,) int32 for x of shape (B, L, d), not together with ``residual``: the rows
     [start, start + len) of each sequence are its tokens (start defaults to 0); it has one group per group end among
     them, the last group taking every token from its first row on; output rows past the groups are zero.
+    ``key_bits`` with ``group_counts`` (``pack_key_bits``, ``side_token_counts``), instead of seq_lens: the same for a
+    mask of any shape -- a group sums its valid rows.
     The result has the weight's dtype when that is 16 bit, else fp32, as torch promotes the reference code."""
     if not (x.is_cuda and weight.is_cuda):
         raise RuntimeError("x and weight must be on a ROCm device: this path has no CPU implementation")
@@ -505,6 +525,16 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, group: in
             a.seq_starts = seq_starts.data_ptr()
     elif seq_starts is not None:
         raise ValueError("seq_starts needs seq_lens")
+    if key_bits is not None or group_counts is not None:
+        need = KEY_BITS_FRONT + (rows + 31) // 32
+        if (key_bits is None or group_counts is None or group <= 1 or seq_lens is not None or residual is not None
+                or key_bits.dtype != torch.int32 or key_bits.dim() != 2 or key_bits.shape[0] != batches or key_bits.shape[1] < need
+                or key_bits.device != x.device or not key_bits.is_contiguous()
+                or group_counts.dtype != torch.int32 or group_counts.shape != (batches,) or group_counts.device != x.device
+                or not group_counts.is_contiguous()):
+            raise ValueError(f"key_bits (B, >= {need}) int32 and group_counts (B,) int32 go together, contiguous on the device "
+                             "of x, with group > 1 and without seq_lens or residual")
+        a.key_bits, a.key_bits_stride, a.group_counts = key_bits.data_ptr(), key_bits.shape[1], group_counts.data_ptr()
     total = None
     if r2 is not None:
         total = torch.empty(x.shape, dtype=x.dtype, device=x.device)
