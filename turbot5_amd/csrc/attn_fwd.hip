@@ -754,16 +754,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     v8 qn[RUNS ? KS : 1];
     auto prefetch_q = [&](int q_tile) {
         if constexpr (RUNS) {
+            // (unconditional: past the last q tile of the run it reads that one again, a lane past the last row reads
+            // the last row -- such rows are computed and not stored; a conditional load makes the compiler merge
+            // register sets at the loop's back edge, behind a wait for the load it has just issued)
             int first, end;
-            qtile_rows(q_tile, first, end);
-            const int row = first + wave * 32 + lr;
+            qtile_rows(min(q_tile, qt_last - 1), first, end);
+            const int row = max(0, min(first + wave * 32 + lr, end - 1));
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) qn[s][e] = (T)0.0f;
-                if (q_tile < qt_last && row < end)
-                    qn[s] = *reinterpret_cast<const v8*>(qp + (int64_t)row * p.q_sr + 16 * s + 8 * hh);
-            }
+            for (int s = 0; s < KS; ++s)
+                qn[s] = *reinterpret_cast<const v8*>(qp + (int64_t)row * p.q_sr + 16 * s + 8 * hh);
         }
     };
     f32x4 qraw[F32 ? D / 4 : 1];
@@ -1529,6 +1528,16 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if constexpr (CURSOR) dma_next(false); else dma_tile(3, false);
     }
 
+    // End of a step: everything but the last two steps' requests has landed.  RUNS: the first two steps of a q tile
+    // may also leave the row stores of the q tile before it in flight (2 * DT store instructions per wavefront, issued
+    // after the requests that these steps wait for and before their own: requests and stores complete in issue order).
+    int relaxed = 0;
+    auto step_wait = [&]() {
+        if constexpr (RUNS) {
+            if (relaxed > 0) { --relaxed; wait_vmcnt<4 * G::SPW + 2 * DT>(); return; }
+        }
+        wait_vmcnt<4 * G::SPW>();   // everything but the last two steps' requests
+    };
     auto step = [&](int t, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         const int kbuf_next = DMA ? (tbase + t + 1) % NSK : (t + 1) & 1;
         const int vbuf = DMA ? (tbase + t) % NSV : t & 1;
@@ -1554,7 +1563,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (!nx.skip) head_refill = softmax_head(nx, st_next);
         tc = nx;
         if constexpr (DMA) {
-            wait_vmcnt<4 * G::SPW>();   // everything but the last two steps' requests
+            step_wait();
             barrier_lds_only();
         } else {
             if (t + 2 < ntiles) store_tile_k(t & 1);
@@ -1673,7 +1682,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
         tc = nx;
         T5A_PHASE(0);
-        wait_vmcnt<4 * G::SPW>();
+        step_wait();
         barrier_lds_only();
         T5A_PHASE(1);
     };
@@ -1693,7 +1702,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
 
     // rows of the current q tile: normalise, convert, store (and the log-sum-exp when asked for)
-    auto store_rows = [&]() {
+    auto store_rows = [&](const int irow, const int row_end_) {   // (a run stores a q tile's rows after it has moved on)
+        const bool row_ok = irow < row_end_;
         const float l_tot = xhalf_sum(l_run + l_alt);
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         if ((MODE == kDense && p.nsplit > 1) || gsplit) {
@@ -1718,22 +1728,53 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     p.part_m[prow] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f : -INFINITY;
                 }
             }
-        } else if (row_ok && irow >= row_lo) {
+        } else {
+            const bool stored = row_ok && irow >= row_lo;
             T* orow = op + (int64_t)irow * p.o_sr;
+            if constexpr (F32) {
+                if (stored) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+                    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int d0 = 32 * dt + 8 * g + 4 * hh;
-                    if (d0 < D) {
-                        f32x4 x;
+                        for (int g = 0; g < 4; ++g) {
+                            const int d0 = 32 * dt + 8 * g + 4 * hh;
+                            if (d0 < D) {
+                                f32x4 x;
 #pragma unroll
-                        for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
-                        if constexpr (F32) *reinterpret_cast<f32x4*>(orow + d0) = x;
-                        else *reinterpret_cast<v4*>(orow + d0) = __builtin_convertvector(x, v4);
-                    }
+                                for (int tt = 0; tt < 4; ++tt) x[tt] = ot[dt][4 * g + tt] * inv;
+                                *reinterpret_cast<f32x4*>(orow + d0) = x;
+                            }
+                        }
                 }
-            if (p.lse != nullptr && hh == 0) {
+            } else {
+                // A lane holds four elements of every eight of its row, the lane 32 further on the other four.  The
+                // two exchange halves, so that each stores 16 contiguous bytes per instruction: half as many store
+                // instructions (2 600 -> 1 500 cycles for the rows of a q tile).  Going on to 64 contiguous bytes
+                // per row (a second exchange between lanes 16 apart) changed nothing.
+                typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        if (32 * dt + 16 * k < D) {
+                            f32x4 xa, xb;
+#pragma unroll
+                            for (int tt = 0; tt < 4; ++tt) {
+                                xa[tt] = ot[dt][8 * k + tt] * inv;
+                                xb[tt] = ot[dt][8 * k + 4 + tt] * inv;
+                            }
+                            const u32x2 a = __builtin_bit_cast(u32x2, __builtin_convertvector(xa, v4));
+                            const u32x2 b2 = __builtin_bit_cast(u32x2, __builtin_convertvector(xb, v4));
+                            // (lanes 32..63 of the first operand trade places with lanes 0..31 of the second)
+                            const auto s0 = __builtin_amdgcn_permlane32_swap(a[0], b2[0], false, false);
+                            const auto s1 = __builtin_amdgcn_permlane32_swap(a[1], b2[1], false, false);
+                            const u32x4 piece = {s0[0], s1[0], s0[1], s1[1]};   // elements 32 dt + 16 k + 8 hh .. + 7
+                            if (stored) *reinterpret_cast<u32x4*>(orow + 32 * dt + 16 * k + 8 * hh) = piece;
+                        }
+                    }
+            }
+            if (stored && p.lse != nullptr && hh == 0) {
                 const float ln2 = 0.6931471805599453f;
                 p.lse[lse_off + (int64_t)irow * p.lse_sr] = l_tot > 0.f ? (m_run + __builtin_log2f(l_tot)) * ln2 : -INFINITY;
             }
@@ -1741,8 +1782,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
 
     T5A_STAMP(3);
-    if constexpr (RUNS) prefetch_q(qt + 1);
     bool interior = first_interior;   // the current q tile's classes hold for any q tile away from the ends of the sequence
+    if constexpr (RUNS) prefetch_q(qt + 1);
     for (;;) {
         int t = 0;
         while (t < ntiles) {
@@ -1774,29 +1815,43 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         T5A_STAMP(trace_slot); ++trace_slot;
         T5A_PHASE_STORE();
         if constexpr (!RUNS) {
-            store_rows();
+            store_rows(irow, row_end);
             break;
         } else {
             // ------------------------------------------------------------ next q tile of the run
             // Its first tiles are in the rings already or on their way (the steps above requested them), the LUT
             // stays, its Q rows were requested a q tile ago.  What is left of a work item's set-up: the geometry
             // and the first score product.
-            if (qt + 1 >= qt_last) { store_rows(); break; }
+            if (qt + 1 >= qt_last) { store_rows(irow, row_end); break; }
+            // The Q rows come through ordinary loads, a q tile ahead.  The compiler copies the freshly requested
+            // registers into the ones the loop carries at the loop's back edge, behind a wait for "nothing outstanding":
+            // a full round trip to memory (2 300 cycles) when the request is the last thing the switch does.  So the
+            // switch reads the rows it has, requests the next ones at once, and does everything else -- stores,
+            // geometry, first product -- while they are on their way.
 #pragma unroll
             for (int s = 0; s < KS; ++s) qf[s] = qn[s];
-            store_rows();
-            ++qt;
-            tbase += ntiles;
-            set_qtile(qt);
-            iw0 = i0 + wave * 32; iw1 = iw0 + 31; irow = iw0 + lr; row_ok = irow < row_end;
-            set_positions();
-            prefetch_q(qt + 1);
             if (!exact) {
 #pragma unroll
                 for (int s = 0; s < KS; ++s)
 #pragma unroll
                     for (int e = 0; e < 8; ++e) qf[s][e] = (T)((float)qf[s][e] * p.c1);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            prefetch_q(qt + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            // (a wavefront none of whose rows is stored issues no store at all)
+            relaxed = __builtin_amdgcn_ballot_w64(row_ok && irow >= row_lo) != 0 ? 2 : 0;
+            store_rows(irow, row_end);
+            ++qt;
+            tbase += ntiles;
+            set_qtile(qt);
+            iw0 = i0 + wave * 32; iw1 = iw0 + 31; irow = iw0 + lr; row_ok = irow < row_end;
+            set_positions();
+            // away from the ends of the sequence every q tile of the local pattern has the same classes
+            const bool was_interior = interior;
+            interior = is_interior();
+            if (!(interior && was_interior)) fill_classes();
+            tc = classify(0);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -1805,11 +1860,6 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             side_cur = 0; cb_cur = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) cm[r] = 0.f;
-            // away from the ends of the sequence every q tile of the local pattern has the same classes
-            const bool was_interior = interior;
-            interior = is_interior();
-            if (!(interior && was_interior)) fill_classes();
-            tc = classify(0);
             if (tc.side != 0) refill_cm(tc.side);
             head_refill = false;
             if (!tc.skip) {
