@@ -488,7 +488,8 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
     elif name == "splitk":
         qd, kc, vc = splitk_inputs(torch, dev)
         f = lambda: ops.flash_decoding_attention(qd, kc, vc, None, 1.0)  # noqa: E731
-        fl = 4.0 * 64 * 12 * 8192 * 64
+        fl = None      # HBM-bound: the K and V rows are read once (2 tensors x 64 x 12 x 8192 x 64 bf16)
+        nbytes = 2.0 * 64 * 12 * 8192 * 64 * 2
     elif name in ("varlen", "varlen_causal"):
         lens, cu, q, k, v, table = varlen_inputs(torch, dev)
         causal = name.endswith("causal")
@@ -498,8 +499,12 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
     else:
         raise SystemExit(f"unknown leg {name!r}")
     _, ms = time_kernel(torch, f, steps, warmup)
-    out = {"leg": name, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
-           "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    if fl is None:
+        out = {"leg": name, "kernel_ms": round(ms, 5), "gbytes_per_s": round(nbytes / ms / 1e6, 1),
+               "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    else:
+        out = {"leg": name, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
+               "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
     if timeline:
         out["timeline"] = read_timeline(torch, f)
     return out
