@@ -1693,6 +1693,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const unsigned long long bad = (cls_skip | cls_mask) >> t;
             return min(bad != 0 ? (int)__builtin_ctzll(bad) : 64, ntiles - t);
         }
+        if (TG && t >= seg_nt[0]) {
+            // side tiles: none is skipped and only a last, partial one needs a mask -- no need to classify sixteen
+            // tiles one by one (some fifty scalar instructions each) to find that out
+            return max(0, min(ntiles, seg_nt[0] + seg_end[1] / BN) - t);
+        }
         int n = 0;
         for (; t + n < ntiles; ++n) {
             const TileClass c = classify(t + n);
