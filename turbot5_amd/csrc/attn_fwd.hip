@@ -434,8 +434,10 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     } else {
         // unsigned arithmetic: the divisions are scalar code on every workgroup's critical path
         const unsigned entry = RUNS ? (unsigned)run_next : (unsigned)w;
-        unsigned bh = entry / (unsigned)p.tiles_per_seq;
-        qt = (int)(entry - bh * (unsigned)p.tiles_per_seq);
+        // (q tiles per sequence are a power of two for the usual lengths: a shift instead of forty instructions)
+        const unsigned tps = (unsigned)p.tiles_per_seq;
+        unsigned bh = (tps & (tps - 1)) == 0 ? entry >> __builtin_ctz(tps | 0x80000000u) : entry / tps;
+        qt = (int)(entry - bh * tps);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
         if (MODE == kBlock && p.nsplit > 1 && w >= p.block_items) {
             // block pattern, behind the block items: key split `split` of the global rows of one (batch, head) --
@@ -560,7 +562,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
     auto set_qtile = [&](int q_tile) {
         if (MODE == kBlock && !gsplit) {
-            blk = q_tile / tpb;
+            blk = tpb == 1 ? q_tile : q_tile / tpb;   // (a division is some forty scalar instructions)
             i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
             row_end = min(Mseq, (blk + 1) * p.block_len);
             seg_start[1] = blk * p.block_len;
@@ -581,7 +583,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // first row and end of the rows of any q tile of this (batch, head)
     auto qtile_rows = [&](int q_tile, int& first, int& end) {
         if (MODE == kBlock) {
-            const int bk = q_tile / tpb;
+            const int bk = tpb == 1 ? q_tile : q_tile / tpb;
             first = bk * p.block_len + (q_tile - bk * tpb) * BM;
             end = min(Mseq, (bk + 1) * p.block_len);
         } else {
@@ -1109,6 +1111,18 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto fill_classes = [&]() {
         cls_skip = cls_mask = cls_lut = cls_right = 0;
         if (!cls_bits) return;
+        if (!(BITS && kbits != nullptr)) {
+            // lane t classifies tile t: some fifty vector instructions for all tiles together instead of as many
+            // scalar ones per tile, in a place where nothing else issues beside them (with validity bit sets the
+            // look-ups would become vector loads, which wait for the tile requests: those go tile by tile)
+            const TileClass c = classify_sparse(lane);
+            const bool in = lane < ntiles;
+            cls_skip = __builtin_amdgcn_ballot_w64(in && c.skip);
+            cls_mask = __builtin_amdgcn_ballot_w64(in && c.need_mask);
+            cls_lut = __builtin_amdgcn_ballot_w64(in && c.use_lut);
+            cls_right = __builtin_amdgcn_ballot_w64(in && c.side == 2);
+            return;
+        }
         for (int t = 0; t < ntiles; ++t) {
             const TileClass c = classify_sparse(t);
             const unsigned long long bit = 1ull << t;
@@ -1165,10 +1179,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
 
     // Query positions in each segment's bias geometry, once per q tile (they take integer divisions by run-time
     // values, some forty instructions each: not something for every tile): the wavefront's range and this lane's own.
+    const int aux_shift = (TG && p.aux > 0 && (p.aux & (p.aux - 1)) == 0) ? __builtin_ctz((unsigned)p.aux) : -1;
     auto position_of = [&](int kind, int row) {
         if (kind == 0) return row + P;
-        if (kind == 1) return row % p.block_len + p.aux;
-        return min(row / p.aux, n_side - 1);   // trailing tokens past the last full block join it
+        // (the rows of a q tile lie in block blk: no division; a row past the block's end is never stored)
+        if (kind == 1) return (MODE == kBlock && !gsplit) ? row - blk * p.block_len + p.aux : row % p.block_len + p.aux;
+        // (side blocks of 2^k tokens, the usual case: a shift instead of a division)
+        const int side = aux_shift >= 0 ? row >> aux_shift : row / p.aux;
+        return min(side, n_side - 1);   // trailing tokens past the last full block join it
     };
     constexpr bool POS_CACHE = MODE == kBlock || TG;   // (the other patterns' positions are row + P)
     auto set_positions = [&]() {
