@@ -192,7 +192,7 @@ __global__ __launch_bounds__(SK_THREADS) void splitk_partial_kernel(const SplitK
 
 // Merge over splits, one wavefront per output row.  The splits' log-sum-exps and weights are read with one
 // lane per split (not one after the other), the weights go through LDS, and the weighted sum over the splits
-// runs four splits at a time so that their loads are in flight together: with 40 and more splits the serial
+// runs eight splits at a time so that their loads are in flight together: with 40 and more splits the serial
 // version spent its time waiting for one load after the other.
 template <typename T, int D>
 __global__ __launch_bounds__(64) void splitk_merge_kernel(const SplitKParams p) {
@@ -201,8 +201,16 @@ __global__ __launch_bounds__(64) void splitk_merge_kernel(const SplitKParams p) 
     const int m = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int lane = threadIdx.x;
     const int64_t base = (((int64_t)b * p.H + h) * p.S) * p.M + m;   // + s * M
-    float gm = -INFINITY;
-    for (int s = lane; s < p.S; s += 64) gm = fmaxf(gm, p.part_m[base + (int64_t)s * p.M]);
+    // The kernel is a chain of dependent loads for a few KB of data, so what it costs is round trips to memory:
+    // a lane's first split is read once (maximum and sum of exponentials together) and kept, and the partial rows
+    // are fetched eight splits at a time.
+    float m_own = -INFINITY, l_own = 0.f;
+    if (lane < p.S) {
+        m_own = p.part_m[base + (int64_t)lane * p.M];
+        l_own = p.part_l[base + (int64_t)lane * p.M];
+    }
+    float gm = m_own;
+    for (int s = lane + 64; s < p.S; s += 64) gm = fmaxf(gm, p.part_m[base + (int64_t)s * p.M]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) gm = fmaxf(gm, __shfl_xor(gm, o, 64));
     auto weight = [&](int s) {
@@ -212,7 +220,7 @@ __global__ __launch_bounds__(64) void splitk_merge_kernel(const SplitKParams p) 
     };
     float wsum = 0.f;
     for (int s = lane; s < p.S; s += 64) {
-        const float w = weight(s);
+        const float w = s == lane ? (l_own > 0.f ? l_own * __expf(m_own - gm) : 0.f) : weight(s);
         if (s < MAXS) s_w[s] = w;
         wsum += w;
     }
@@ -220,18 +228,20 @@ __global__ __launch_bounds__(64) void splitk_merge_kernel(const SplitKParams p) 
     for (int o = 32; o > 0; o >>= 1) wsum += __shfl_xor(wsum, o, 64);
     __syncthreads();
     T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)m * p.o_sr;
+    const int cached = p.S < MAXS ? p.S : MAXS;
     for (int d = lane; d < D; d += 64) {
         float val = 0.f;
         int s = 0;
-        for (; s + 4 <= p.S && s + 4 <= MAXS; s += 4) {
-            float x[4];
+        for (; s < cached; s += 8) {   // (MAXS is a multiple of 8)
+            float x[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) x[i] = p.part_o[(base + (int64_t)(s + i) * p.M) * D + d];
+            for (int i = 0; i < 8; ++i) x[i] = s + i < cached ? p.part_o[(base + (int64_t)(s + i) * p.M) * D + d] : 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) val = s_w[s + i] > 0.f ? fmaf(x[i], s_w[s + i], val) : val;   // an empty split's row may hold anything
+            for (int i = 0; i < 8; ++i)   // an empty split's row may hold anything
+                if (s + i < cached) val = s_w[s + i] > 0.f ? fmaf(x[i], s_w[s + i], val) : val;
         }
-        for (; s < p.S; ++s) {
-            const float w = s < MAXS ? s_w[s] : weight(s);
+        for (s = cached; s < p.S; ++s) {
+            const float w = weight(s);
             if (w > 0.f) val = fmaf(p.part_o[(base + (int64_t)s * p.M) * D + d], w, val);
         }
         op[d] = SkLoad<T>::cvt(wsum > 0.f ? val / wsum : 0.f);
