@@ -1711,6 +1711,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const unsigned long long bad = (cls_skip | cls_mask) >> t;
             return min(bad != 0 ? (int)__builtin_ctzll(bad) : 64, ntiles - t);
         }
+        // window tiles: a wavefront's plain ones (every key inside the window of every row) start within an interval
+        // of 2 * window - 94 keys; four fast steps take five plain tiles in a row, so narrow windows have none
+        if (TG && t < seg_nt[0] && 2 * p.block_len - 94 < 5 * BN) return 0;
         if (TG && t >= seg_nt[0]) {
             // side tiles: none is skipped and only a last, partial one needs a mask -- no need to classify sixteen
             // tiles one by one (some fifty scalar instructions each) to find that out
