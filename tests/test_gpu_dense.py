@@ -509,3 +509,34 @@ def test_raw_ctypes_binding_as_a_reference_maintainer_would_write_it(gpu_device)
         want = O.dense_attention(q, k, v, table, causal, 1.0)
         assert (o.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
         assert (lse.cpu() - O.dense_lse(q, k, table, causal, 1.0)).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+def test_output_in_token_major_layout_with_guard_rows(gpu_device, dt, D):
+    """The write-back stores rows in 16-byte pieces (after an exchange between the halves of a wavefront): output in
+    (B, M, H, D) layout through the C ABI, a ragged number of rows, every head dimension; rows and heads that do not
+    belong to the call keep their fill value."""
+    import ctypes as C
+    from turbot5_amd import _lib as L
+    from turbot5_amd import ops
+    B, H, M, N = 2, 3, 77, 150
+    q, k, v = (rnd(B, H, n, D, seed=300 + i, dtype=dt).to(gpu_device) for i, n in enumerate((M, N, N)))
+    table = rnd(32, H, seed=303, scale=1.0).to(gpu_device)
+    fill = 123.0
+    buf = torch.full((B, M + 3, H + 1, D), fill, device=gpu_device, dtype=dt)      # guard rows and a guard head
+    o = buf[:, :M, :H].permute(0, 2, 1, 3)                                          # (B, H, M, D) view, rows H + 1 heads apart
+    a = L.T5ADenseArgs()
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+    a.q_strides, a.k_strides, a.v_strides, a.o_strides = (ops._strides3(t) for t in (q, k, v, o))
+    a.dtype = {torch.bfloat16: L.T5A_BF16, torch.float16: L.T5A_F16, torch.float32: L.T5A_F32}[dt]
+    a.B, a.H, a.M, a.N, a.D = B, H, M, N, D
+    a.causal, a.sm_scale = 0, 1.0
+    a.bias, keep = ops._bias_struct(table, H, 32, 128, q)
+    L.check(L.load().t5a_fwd_dense(C.byref(a), ops._stream(q)))
+    torch.cuda.synchronize()
+    want = O.dense_attention(q.cpu(), k.cpu(), v.cpu(), table.cpu(), False, 1.0)
+    got = o.float().cpu()
+    assert (got - want).abs().max().item() <= TOL[dt]
+    host = buf.float().cpu()
+    assert (host[:, M:] == fill).all() and (host[:, :, H] == fill).all()
