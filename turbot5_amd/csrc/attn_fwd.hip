@@ -303,11 +303,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     constexpr bool DENSE = MODE == kDense || MODE == kPacked;   // one key segment starting at key 0
     constexpr bool LOCAL = MODE == kLocal || MODE == kLocalWide;   // sliding window, one segment
     constexpr bool TG = MODE == kTGlobal || MODE == kTGlobalBits;   // sliding window and side tokens
+    constexpr bool BLOCK = MODE == kBlock || MODE == kBlockBits;    // own block and leading global tokens
     // Sparse patterns, LDS-DMA geometries: a work item is a RUN of consecutive q tiles of one (batch, head).  Their
     // key tiles form one stream through the LDS rings (the requests for the next q tile's first tiles go out during
     // the last steps of the current one) and the distance LUT is built once per run; a q tile of a sparse pattern
     // is only a few steps long, so that its set-up would otherwise cost as much as its steps.
-    constexpr bool RUNS = (MODE == kLocal || MODE == kBlock) && G::DMA;
+    constexpr bool RUNS = (MODE == kLocal || BLOCK) && G::DMA;
     constexpr bool CURSOR = MODE == kLocal && G::DMA;   // one segment: the requests of a run advance cursors
     // head_dim 64, 16-bit types: the Q rows are staged through LDS by LDS-DMA as well (see the prologue)
     constexpr bool QDMA = G::DMA && D == 64;
@@ -363,7 +364,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const unsigned wi = (ga + (k - level * gx)) * tps + level;
         if (wi < lo || wi >= hi) return;
         w = (int)wi;
-    } else if (MODE == kBlock && p.nsplit > 1) {
+    } else if (BLOCK && p.nsplit > 1) {
         // the key splits of the global rows are the longer items: they take the first workgroup ids, so that they
         // start first and the block items fill in around them; the block items follow in per-XCD slices
         const int n_split = p.total_items - p.block_items;
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (RUNS) {
         run_next = w * p.run_len;
         run_left = min(p.run_len, p.tiles_per_seq * p.H * p.B - run_next);
-        if (MODE == kBlock && p.nsplit > 1 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
+        if (BLOCK && p.nsplit > 1 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
     }
     for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
@@ -439,7 +440,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         unsigned bh = (tps & (tps - 1)) == 0 ? entry >> __builtin_ctz(tps | 0x80000000u) : entry / tps;
         qt = (int)(entry - bh * tps);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
-        if (MODE == kBlock && p.nsplit > 1 && w >= p.block_items) {
+        if (BLOCK && p.nsplit > 1 && w >= p.block_items) {
             // block pattern, behind the block items: key split `split` of the global rows of one (batch, head) --
             // its first G rows attend all keys, standard bias; the partial results are merged by a second kernel
             gsplit = true;
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
         // masks of any shape: the caller counts the block ENDs among the valid tokens
         if (TG && p.side_counts != nullptr) n_side = max(0, min(p.n_side, p.side_counts[b]));
-        if (MODE == kBlock && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
+        if (BLOCK && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -488,9 +489,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     T* op = reinterpret_cast<T*>(p.o) + o_off;
     // sparse patterns, masks of any shape: validity of this sequence's tokens as a bit set (the global rows'
     // key splits of the block pattern attend every key, as in the reference)
-    // (local and transient-global patterns: the host sends such batches to instantiations of their own, kLocalWide
-    // and kTGlobalBits, so that the ones for batches without holes carry none of this)
-    constexpr bool BITS = MODE == kLocalWide || MODE == kBlock || MODE == kTGlobalBits;
+    // (the host sends such batches to instantiations of their own -- kLocalWide, kBlockBits, kTGlobalBits -- so that
+    // the ones for batches without holes carry none of this)
+    constexpr bool BITS = MODE == kLocalWide || MODE == kBlockBits || MODE == kTGlobalBits;
     const unsigned* kbits = (BITS && p.key_bits != nullptr && !gsplit) ? p.key_bits + (int64_t)b * p.key_bits_stride : nullptr;
     // validity of the tokens pos0 .. pos0 + 63, bit e = token pos0 + e (wavefront-uniform: scalar loads)
     auto token_bits = [&](int pos0) {
@@ -505,8 +506,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     const int qt_last = qt + qt_count;   // one past the last q tile of this pass
     // query rows of the current q tile: [i0, row_end); rows below row_lo are computed but not stored
     int i0 = 0, row_end = 0, row_lo = 0, blk = 0;
-    const int tpb = MODE == kBlock ? (p.block_len + BM - 1) / BM : 1;   // q tiles per block (block pattern)
-    if (MODE == kBlock && !gsplit) row_lo = p.aux;   // the first G rows belong to the key-split items / the global-query pass
+    const int tpb = BLOCK ? (p.block_len + BM - 1) / BM : 1;   // q tiles per block (block pattern)
+    if (BLOCK && !gsplit) row_lo = p.aux;   // the first G rows belong to the key-split items / the global-query pass
     const int P = p.align_end ? Nseq - Mseq : -key0;   // query position minus row index, in this item's key numbering
 
     // ---------------------------------------------------------------- key segments
@@ -536,11 +537,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             seg_ksr[1] = (int)p.sk_sr * ES; seg_vsr[1] = (int)p.sv_sr * ES;
             seg_end[1] = n_side; seg_lend[1] = n_side; seg_kind[1] = 2;
         }
-    } else if (MODE == kBlock && !gsplit) {
+    } else if (BLOCK && !gsplit) {
         nseg = 2;
         seg_end[0] = p.aux; seg_kind[0] = 1;
         seg_lend[1] = Nseq;
-    } else if (MODE == kBlock) {
+    } else if (BLOCK) {
         seg_end[0] = Nseq;   // one segment: this split's keys, query i at position i (P = -key0)
     }
     // The part of the geometry that changes from one q tile to the next.  RUNS: every q tile of the run has the
@@ -561,7 +562,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         span = blk == 0 ? 0 : max(0, p.block_len - p.aux - head);
     };
     auto set_qtile = [&](int q_tile) {
-        if (MODE == kBlock && !gsplit) {
+        if (BLOCK && !gsplit) {
             blk = tpb == 1 ? q_tile : q_tile / tpb;   // (a division is some forty scalar instructions)
             i0 = blk * p.block_len + (q_tile - blk * tpb) * BM;
             row_end = min(Mseq, (blk + 1) * p.block_len);
@@ -582,7 +583,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
     // first row and end of the rows of any q tile of this (batch, head)
     auto qtile_rows = [&](int q_tile, int& first, int& end) {
-        if (MODE == kBlock) {
+        if (BLOCK) {
             const int bk = tpb == 1 ? q_tile : q_tile / tpb;
             first = bk * p.block_len + (q_tile - bk * tpb) * BM;
             end = min(Mseq, (bk + 1) * p.block_len);
@@ -593,8 +594,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     };
     set_qtile(qt);
     if constexpr (RUNS) {
-        if (MODE == kBlock && gsplit) { seg_nt[0] = (Nseq + BN - 1) / BN; seg_nt[1] = 0; }
-        else if (MODE == kBlock) { seg_nt[0] = (p.aux + BN - 1) / BN; seg_nt[1] = (p.block_len + BN - 1) / BN; }
+        if (BLOCK && gsplit) { seg_nt[0] = (Nseq + BN - 1) / BN; seg_nt[1] = 0; }
+        else if (BLOCK) { seg_nt[0] = (p.aux + BN - 1) / BN; seg_nt[1] = (p.block_len + BN - 1) / BN; }
         else { seg_nt[0] = (BM + 2 * p.block_len - 2 + BN - 1) / BN; seg_nt[1] = nseg > 1 ? (n_side + BN - 1) / BN : 0; }
     } else {
         seg_nt[0] = max(0, seg_end[0] - seg_start[0] + BN - 1) / BN;
@@ -603,7 +604,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // an even number of tiles per q tile keeps the two score buffers of the pipeline in step from one q tile of a
     // run to the next (the extra tile lies past its segment's end and is skipped)
     // (the block pattern's q tiles are too short for fast steps anyway: no rounding there)
-    if (RUNS && MODE != kBlock && ((seg_nt[0] + seg_nt[1]) & 1)) {   // (no run-time index: that would move the array to scratch memory)
+    if (RUNS && !BLOCK && ((seg_nt[0] + seg_nt[1]) & 1)) {   // (no run-time index: that would move the array to scratch memory)
         if (nseg > 1) seg_nt[1] += 1; else seg_nt[0] += 1;
     }
     const int ntiles = seg_nt[0] + seg_nt[1];   // tiles of one q tile
@@ -614,7 +615,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     for (int sg = 0; sg < 2; ++sg) {
         // rows at or past this read as zero.  RUNS: one descriptor per tensor for the whole run -- all the keys of
         // the (batch, head); what a q tile must not see of them is masked
-        const int rows = RUNS ? (sg == 0 || MODE == kBlock ? Nseq : n_side) : min(seg_lend[sg], seg_end[sg]);
+        const int rows = RUNS ? (sg == 0 || BLOCK ? Nseq : n_side) : min(seg_lend[sg], seg_end[sg]);
         const unsigned kb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_ksr[sg] + D * ES : 0u;
         const unsigned vb = rows > 0 ? (unsigned)(rows - 1) * (unsigned)seg_vsr[sg] + D * ES : 0u;
         seg_krs[sg] = make_rsrc(seg_k[sg], kb);
@@ -636,7 +637,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             sg = t >= seg_nt[0] ? 1 : 0;
             const int ts = t - (sg ? seg_nt[0] : 0);
             // (a scalar division costs some forty instructions, and this runs for every request)
-            if (MODE == kBlock) j0 = sg ? (tpb == 1 ? q_tile : q_tile / tpb) * p.block_len + ts * BN : ts * BN;
+            if (BLOCK) j0 = sg ? (tpb == 1 ? q_tile : q_tile / tpb) * p.block_len + ts * BN : ts * BN;
             else j0 = sg ? ts * BN : q_tile * BM - p.block_len + 1 + ts * BN;
             return q_tile < qt_last;
         } else {
@@ -1056,7 +1057,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // Validity of the 64 keys of a tile as the pattern's mask sees them (bit e = key j0 + e); kbits != nullptr.
     auto tile_valid = [&](int sg, int j0) {
         if (TG && sg == 1) return ~0ull;   // side tokens: the count of them is the mask
-        if (MODE != kBlock) return token_bits(j0);
+        if (!BLOCK) return token_bits(j0);
         // block pattern: list column c < block_len of [G global tokens | own block] takes the bit of token
         // blk * block_len + c (the reference's mask layout, attentions.py:722-732)
         if (sg == 0) return token_bits(blk * p.block_len + j0);            // global key j is column j
@@ -1073,7 +1074,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const int kind = (c.sg ? seg_kind[1] : seg_kind[0]);
         const bool win = (c.sg ? seg_win[1] : seg_win[0]) != 0;
         (void)kind;
-        constexpr bool cached = MODE == kBlock || TG;   // positions kept per q tile (set_positions)
+        constexpr bool cached = BLOCK || TG;   // positions kept per q tile (set_positions)
         const int qlo = cached ? (c.sg ? wq_lo[1] : wq_lo[0]) : iw0 + P, qhi = cached ? (c.sg ? wq_hi[1] : wq_hi[0]) : iw1 + P;
         const int rel_min = c.j0 - qhi, rel_max = c.j0 + BN - 1 - qlo;
         c.skip = iw0 >= row_end;                              // wavefront without live rows
@@ -1090,7 +1091,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             c.need_mask = c.need_mask || c.j0 < key_lo;
         }
         if (win && !win_lut) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
-        if (MODE == kBlock && c.sg == 1 && n_valid < Nseq) {
+        if (BLOCK && c.sg == 1 && n_valid < Nseq) {
             int hole_lo, hole_span;
             block_hole(hole_lo, hole_span);
             c.need_mask = c.need_mask || (c.j0 < hole_lo + hole_span && c.j0 + BN > hole_lo);
@@ -1183,12 +1184,12 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto position_of = [&](int kind, int row) {
         if (kind == 0) return row + P;
         // (the rows of a q tile lie in block blk: no division; a row past the block's end is never stored)
-        if (kind == 1) return (MODE == kBlock && !gsplit) ? row - blk * p.block_len + p.aux : row % p.block_len + p.aux;
+        if (kind == 1) return (BLOCK && !gsplit) ? row - blk * p.block_len + p.aux : row % p.block_len + p.aux;
         // (side blocks of 2^k tokens, the usual case: a shift instead of a division)
         const int side = aux_shift >= 0 ? row >> aux_shift : row / p.aux;
         return min(side, n_side - 1);   // trailing tokens past the last full block join it
     };
-    constexpr bool POS_CACHE = MODE == kBlock || TG;   // (the other patterns' positions are row + P)
+    constexpr bool POS_CACHE = BLOCK || TG;   // (the other patterns' positions are row + P)
     auto set_positions = [&]() {
         if constexpr (!POS_CACHE) return;
         const int ir = min(irow, max(row_end - 1, iw0));   // rows past the end are never stored: keep them in range
@@ -1305,7 +1306,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const int jl = c.j0 + 4 * hh - lo;
             // block pattern on a padded sequence: a range of the own block's keys that the rows do not see
             int hole_lo = 0, hole_span = 0;
-            if (MODE == kBlock && c.sg == 1) block_hole(hole_lo, hole_span);
+            if (BLOCK && c.sg == 1) block_hole(hole_lo, hole_span);
             const unsigned hspan = (unsigned)hole_span;
             const int jh = c.j0 + 4 * hh - hole_lo;
             // masks of any shape: this lane's keys of the tile's validity bits, bit `off` below
@@ -1317,7 +1318,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 for (int r = 0; r < 16; ++r) {
                     const int off = 32 * nt + 8 * (r >> 2) + (r & 3);
                     bool keep = (unsigned)(jl + off) < span;
-                    if (MODE == kBlock) keep = keep && !((unsigned)(jh + off) < hspan);
+                    if (BLOCK) keep = keep && !((unsigned)(jh + off) < hspan);
                     if (BITS) keep = keep && ((vm >> off) & 1ull) != 0;
                     st[nt][r] = keep ? st[nt][r] : -INFINITY;
                 }
@@ -1515,7 +1516,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     auto is_interior = [&]() {
         if (BITS && kbits != nullptr) return false;   // (every q tile looks its keys' validity up)
         if (LOCAL) return seg_start[0] >= key_lo && i0 + BM - 1 + p.block_len <= Nseq && i0 + BM <= Mseq;
-        if (MODE == kBlock) return !gsplit && tpb == 1 && blk >= 1 && (blk + 1) * p.block_len <= min(Nseq, n_valid) && i0 + BM <= Mseq;
+        if (BLOCK) return !gsplit && tpb == 1 && blk >= 1 && (blk + 1) * p.block_len <= min(Nseq, n_valid) && i0 + BM <= Mseq;
         return false;
     };
     const bool first_interior = is_interior();
@@ -1939,7 +1940,7 @@ static hipError_t launch_exact(const FwdParams& p, hipStream_t stream) {
         }
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
-    if (MODE == kBlock && p.nsplit > 1)
+    if ((MODE == kBlock || MODE == kBlockBits) && p.nsplit > 1)
         grid = (unsigned)(((p.total_items - p.block_items + 7) / 8) * 8 + ((p.block_items + 7) / 8) * 8);
     if (MODE == kPacked && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
     if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {
@@ -1969,6 +1970,7 @@ static hipError_t launch_mode(const FwdParams& p, int mode, bool causal, hipStre
         case kLocal: return launch_one<T, D, kLocal, false>(p, s);
         case kLocalWide: return launch_one<T, D, kLocalWide, false>(p, s);
         case kBlock: return launch_one<T, D, kBlock, false>(p, s);
+        case kBlockBits: return launch_one<T, D, kBlockBits, false>(p, s);
         case kTGlobal: return launch_one<T, D, kTGlobal, false>(p, s);
         case kTGlobalBits: return launch_one<T, D, kTGlobalBits, false>(p, s);
     }

@@ -25,8 +25,9 @@ struct BucketSpec {
 // kPacked: dense semantics per sequence of a packed batch (cu_seqlens); a separate instantiation, so that
 // the unpacked kernel carries none of its work-item search
 // kLocal: sliding window of at most kMaxLutWindow, folded into the distance LUT; kLocalWide: wider windows, masked
-// per element at their edges, and masks of any shape; kTGlobalBits: transient-global with masks of any shape
-enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLocalWide = 5, kTGlobalBits = 6 };
+// per element at their edges, and masks of any shape; kTGlobalBits, kBlockBits: the transient-global and block
+// patterns with masks of any shape
+enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLocalWide = 5, kTGlobalBits = 6, kBlockBits = 7 };
 // widest sliding window that is folded into the distance LUT (the LUT then spans 2 * (window + 96) distances;
 // 256 keeps it below 12 KB of LDS, so that two workgroups still share a compute unit)
 constexpr int kMaxLutWindow = 256;
