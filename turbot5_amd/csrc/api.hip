@@ -570,7 +570,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
             const int64_t items = (int64_t)p.block_items + (int64_t)p.nsplit * a->H * a->B;
             if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
             p.total_items = (int)items;
-            rc = finish(launch_fwd(p, a->dtype, a->D, a->key_bits != nullptr ? kBlockBits : kBlock, false, s), "t5a_fwd_sparse(block + global rows as key splits)");
+            rc = finish(launch_fwd(p, a->dtype, a->D, (a->key_bits != nullptr || a->seq_lens != nullptr) ? kBlockBits : kBlock, false, s), "t5a_fwd_sparse(block + global rows as key splits)");
             if (rc) return rc;
             SplitKParams m;
             memset(&m, 0, sizeof(m));
@@ -579,7 +579,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
             m.B = a->B; m.H = a->H; m.M = G; m.S = p.nsplit;
             return finish(launch_splitk_merge(m, a->dtype, a->D, s), "t5a_fwd_sparse(block, merge)");
         }
-        rc = finish(launch_fwd(p, a->dtype, a->D, a->key_bits != nullptr ? kBlockBits : kBlock, false, s), "t5a_fwd_sparse(block)");
+        rc = finish(launch_fwd(p, a->dtype, a->D, (a->key_bits != nullptr || a->seq_lens != nullptr) ? kBlockBits : kBlock, false, s), "t5a_fwd_sparse(block)");
         if (rc || a->aux == 0) return rc;
         // the G global queries as a pass of their own: M is clipped to G rows of the same tensors
         FwdParams g = p;

@@ -471,7 +471,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         }
         // masks of any shape: the caller counts the block ENDs among the valid tokens
         if (TG && p.side_counts != nullptr) n_side = max(0, min(p.n_side, p.side_counts[b]));
-        if (BLOCK && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
+        // (padded batches of the block pattern run in the instantiation for masks: the plain one knows n_valid as a constant)
+        if (MODE == kBlockBits && p.len_k != nullptr) n_valid = max(0, min(p.N, p.len_k[b]));
         q_off = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
         k_off = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -1091,7 +1092,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             c.need_mask = c.need_mask || c.j0 < key_lo;
         }
         if (win && !win_lut) c.need_mask = c.need_mask || (rel_max >= p.block_len) || (rel_min <= -p.block_len);
-        if (BLOCK && c.sg == 1 && n_valid < Nseq) {
+        if (MODE == kBlockBits && c.sg == 1 && n_valid < Nseq) {
             int hole_lo, hole_span;
             block_hole(hole_lo, hole_span);
             c.need_mask = c.need_mask || (c.j0 < hole_lo + hole_span && c.j0 + BN > hole_lo);
@@ -1306,7 +1307,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             const int jl = c.j0 + 4 * hh - lo;
             // block pattern on a padded sequence: a range of the own block's keys that the rows do not see
             int hole_lo = 0, hole_span = 0;
-            if (BLOCK && c.sg == 1) block_hole(hole_lo, hole_span);
+            if (MODE == kBlockBits && c.sg == 1) block_hole(hole_lo, hole_span);
             const unsigned hspan = (unsigned)hole_span;
             const int jh = c.j0 + 4 * hh - hole_lo;
             // masks of any shape: this lane's keys of the tile's validity bits, bit `off` below
@@ -1318,7 +1319,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 for (int r = 0; r < 16; ++r) {
                     const int off = 32 * nt + 8 * (r >> 2) + (r & 3);
                     bool keep = (unsigned)(jl + off) < span;
-                    if (BLOCK) keep = keep && !((unsigned)(jh + off) < hspan);
+                    if (MODE == kBlockBits) keep = keep && !((unsigned)(jh + off) < hspan);
                     if (BITS) keep = keep && ((vm >> off) & 1ull) != 0;
                     st[nt][r] = keep ? st[nt][r] : -INFINITY;
                 }
