@@ -19,15 +19,20 @@
  *    of the last failure on the calling thread is t5a_last_error().
  *  - Scores are q.k * sm_scale + bias; the T5 modules pass sm_scale = 1.0.
  *  - Score precision (bf16 and fp16 inputs; the exact_scores field of the dense, varlen and sparse
- *    arguments).  0 (default): the query rows are multiplied by sm_scale * log2(e) and rounded back to the
+ *    arguments takes one of the T5A_SCORES_* values below; fp32 inputs are always exact).
+ *    T5A_SCORES_DEFAULT (0): the query rows are multiplied by sm_scale * log2(e) and rounded back to the
  *    input type before the matrix product, a relative error of 2^-9 (bf16) on every term of a score.
  *    With unscaled T5 scores of deviation 8 (18) the output error against fp32 math on the same inputs is
  *    about 4.5e-2 (1.1e-1) at worst, 3.6 times below that of the reference's 'basic' path run in bf16
- *    (src/turbot5/ops/naive_attention.py:4-23 rounds the scores themselves to bf16).  Non-zero: the query
- *    rows enter the product as they are and the factor is applied to the fp32 result, as the reference's
- *    fused kernel does (src/turbot5/ops/fused_bias_attention.py:323-337); the error stays near 1e-2 (the
- *    rounding of the output) at any score magnitude and the kernels take about 11 % longer at head_dim 64.
- *    fp32 inputs are always exact.
+ *    (src/turbot5/ops/naive_attention.py:4-23 rounds the scores themselves to bf16).
+ *    T5A_SCORES_EXACT (1): the query rows enter the product as they are and the factor is applied to the
+ *    fp32 result, as the reference's fused kernel does (src/turbot5/ops/fused_bias_attention.py:323-337);
+ *    the error stays near 1e-2 (the rounding of the output) at any score magnitude; one more vector
+ *    multiply per score.
+ *    T5A_SCORES_PRESCALED (2): q already holds the query rows times sm_scale * log2(e) -- the caller folded
+ *    the factor into the projection that produced q, in fp32, so that q was rounded to its type once.  The
+ *    kernel applies no factor (sm_scale is not read); accuracy of T5A_SCORES_EXACT at the speed of
+ *    T5A_SCORES_DEFAULT.  This is what the attention modules of this package do.
  *  - The relative-position bias is never materialised: kernels derive
  *    bucket(key_pos - query_pos) from integer positions and read the
  *    (num_buckets, H) table.  Bucket boundaries are computed on the host with
@@ -101,7 +106,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 112
+#define T5A_ABI_VERSION 113
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -123,6 +128,8 @@ int t5a_bucket_lut(int bidirectional, int num_buckets, int max_distance, int32_t
  * unidirectional, else bidirectional.  lse (optional) is (B,H,M) contiguous
  * fp32, natural log of the softmax normaliser (fused_bias_attention.py:358).
  */
+enum { T5A_SCORES_DEFAULT = 0, T5A_SCORES_EXACT = 1, T5A_SCORES_PRESCALED = 2 };
+
 typedef struct t5a_dense_args {
     const void* q; const void* k; const void* v; void* o; float* lse;
     int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3];
@@ -240,11 +247,27 @@ typedef struct t5a_sparse_args {
     const uint32_t* key_bits;
     int64_t key_bits_stride;      /* words per sequence */
     const int32_t* side_counts;   /* TGLOBAL with key_bits: (B) int32, side tokens of each sequence */
+    /* LOCAL (windows up to 256) and BLOCK with 16-bit inputs at head_dim 64 / 128: a work item takes run_len
+     * consecutive q tiles of one (batch, head).  0: the library chooses from the shape and the device's size;
+     * 1..16: this many (tests pin every path with it; results do not depend on it). */
+    int32_t run_len; int32_t reserved;
 } t5a_sparse_args;
 /* words per sequence that key_bits needs (front padding, ceil(L / 32), back padding) */
 int64_t t5a_sparse_key_bits_words(int32_t L, int32_t block_len, int32_t aux);
 int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len, int32_t aux);
 int t5a_fwd_sparse(const t5a_sparse_args* args, t5a_stream_t stream);
+/*
+ * Host-only: the launch plan t5a_fwd_sparse would choose for a shape, without touching the device when
+ * compute_units > 0 (0: ask the current device).  No counterpart in the reference (its sparse modules are torch
+ * code with one fixed blocking, src/turbot5/model/attentions.py:583-638, :788-853).  with_workspace: the call
+ * would pass a workspace of t5a_sparse_workspace_bytes().  run_len as in t5a_sparse_args.
+ * out[0] = q tiles per run, out[1] = work items of the launch, out[2] = how many of them are runs when the
+ * global rows of the block pattern travel in the same launch as key splits (else 0), out[3] = key splits per
+ * (batch, head), out[4] = keys per split, out[5] = q tiles per (batch, head).  Fails (T5A_ERR_LAUNCH) if the plan
+ * would not cover every q tile and every key exactly once.
+ */
+int t5a_sparse_launch_plan(int32_t pattern, int32_t dtype, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len,
+                           int32_t aux, int32_t with_workspace, int32_t compute_units, int32_t run_len, int32_t* out /* 6 */);
 
 /*
  * Flash-decoding split-K forward for few query rows over a long memory.

@@ -145,6 +145,10 @@ CASES = [
     ("T5TransientGlobalAttention", 2, 64, 2, 16, 16, 8, "left"),
     ("T5TransientGlobalAttention", 2, 64, 2, 16, 16, 8, "holes"),
     ("T5TransientGlobalAttention", 1, 96, 3, 16, 32, 16, "right"),
+    # padded batches shorter than one block: full attention under a key mask (attentions.py:752, :691, :722-732)
+    ("T5BlockAttention", 2, 10, 2, 16, 16, 4, "right"),
+    ("T5BlockAttention", 3, 13, 2, 16, 16, 4, "holes"),
+    ("T5BlockAttention", 2, 12, 2, 16, 16, 4, "left"),
 ]
 
 

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import t5_basic as O
-from tests.test_oracle_fixtures import CASES
+from tests.test_oracle_fixtures import CASES, oracle_attention_output
 
 pytestmark = pytest.mark.gpu
 
@@ -56,7 +56,16 @@ def test_module_matches_reference_vectors(gpu_device, name, c):
     else:
         rows = mask.bool()
     err = (got - c["out"]).abs()[rows].max().item()
-    assert err <= 2e-4, f"{name}: max-abs {err}"
+    assert err <= 2e-4, f"{name}: max-abs {err}"   # (the output projection adds its own fp32 rounding)
+    # the attention op itself, at the input of the output projection, holds the 1e-4 bar of an fp32 attention op:
+    # against the oracle's restatement of the module's op, which the CPU suite matches to the reference's vectors
+    # (tests/test_oracle_fixtures.py) to 1e-6
+    attn = seen["attn"].cpu().view(B, L, H, D).transpose(1, 2)
+    want = oracle_attention_output(name, c)
+    tok = mask.bool()[:, None, :, None].expand_as(want)
+    assert torch.isfinite(attn[tok]).all()
+    err_op = (attn - want)[tok].abs().max().item()
+    assert err_op <= 1e-4, f"{name}: attention op max-abs {err_op}"
 
 
 # ------------------------------------------------------------------------------------------------
@@ -214,25 +223,38 @@ def test_lut_cache_is_not_poisoned_by_calls_that_never_launch(gpu_device):
 # ------------------------------------------------------------------------------------------------
 # accuracy at the score magnitudes of unscaled T5 attention
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("exact", [False, True])
+@pytest.mark.parametrize("exact", [False, True, "prescaled"])
 @pytest.mark.parametrize("scale", [1.0, 1.5])
 @pytest.mark.parametrize("kind", ["dense", "causal", "varlen", "local", "block", "tglobal"])
 def test_bf16_accuracy_at_large_scores(gpu_device, kind, scale, exact):
     """T5 does not scale its scores: with q, k ~ N(0, scale^2) at head_dim 64 they have a deviation of
-    8 * scale^2 (8 and 18 here, against 2 for the 0.5 * randn inputs of the other tests).  Error against the
-    fp32 oracle on the same bf16-rounded inputs, max-abs over outputs of order 1:
-      default          <= 6e-2 (deviation 8), <= 1.5e-1 (deviation 18): the rounding of Q * log2(e) to bf16; and
-                       never above the error of the reference's literal bf16 'basic' path
-                       (naive_attention.py:4-23: scores rounded to bf16 before an fp32 softmax)
-      exact_scores     <= 2e-2 at either magnitude: only the roundings of the probabilities and of the output."""
+    sigma = 8 * scale^2 (8 and 18 here, against 2 for the 0.5 * randn inputs of the other tests).  Error against
+    the fp32 oracle on the same bf16-rounded inputs, max-abs over outputs of order 1:
+      exact_scores, prescaled q   <= 2e-2 at either magnitude: only the roundings of the probabilities and of the
+                       output are left (prescaled: the oracle gets the rows the kernel gets, divided by log2 e).
+      default          the kernel rounds Q * log2(e) to bf16 once more: a relative error of at most 2^-9, uniform,
+                       on each of the 64 terms of a score, so a score is off by tau = sigma * 2^-9 / sqrt(3)
+                       (standard deviation).  An output suffers most where a row's weight sits on two keys: it
+                       moves by p (1 - p) (ds1 - ds2) (v1 - v2) <= 1/4 * (z sqrt(2) tau) * dv, with z = 4.5
+                       deviations (the worst of the 1e5 outputs here) and dv = 4 (two N(0,1) values that far
+                       apart), on top of 1e-2 for the rounding of the output itself.  That is 0.067 at
+                       deviation 8 and 0.139 at 18 -- a requirement derived from the one extra rounding, not a
+                       measurement; the kernel must also never be worse than the reference's literal bf16
+                       'basic' path (naive_attention.py:4-23: scores rounded to bf16 before an fp32 softmax)."""
     from turbot5_amd import ops
-    bound = 2e-2 if exact else (6e-2 if scale == 1.0 else 1.5e-1)
+    sigma = 8.0 * scale * scale
+    tau = sigma * 2.0 ** -9 / math.sqrt(3.0)
+    bound = 2e-2 if exact else 1e-2 + 0.25 * (4.5 * math.sqrt(2.0) * tau) * 4.0
     g = torch.Generator().manual_seed(11)
     B, H, L, D = 2, 2, 512, 64
     q, k = ((scale * torch.randn(B, H, L, D, generator=g)).to(torch.bfloat16) for _ in range(2))
     v = torch.randn(B, H, L, D, generator=g).to(torch.bfloat16)
     table = torch.randn(32, H, generator=g)
     dq, dk, dv, dt = (t.to(gpu_device) for t in (q, k, v, table))
+    if exact == "prescaled":
+        # the rows as a projection with log2(e) folded in hands them over: scaled in fp32, rounded once
+        qs = (q.float() * LOG2E).to(torch.bfloat16)
+        dq, q = qs.to(gpu_device), qs.float() / LOG2E
     literal = None
     if kind in ("dense", "causal"):
         causal = kind == "causal"
@@ -242,7 +264,8 @@ def test_bf16_accuracy_at_large_scores(gpu_device, kind, scale, exact):
     elif kind == "varlen":
         cu = torch.tensor([0, 300, 812, 1024], dtype=torch.int32)
         qp, kp, vp = (t.transpose(1, 2).reshape(B * L, H, D) for t in (q, k, v))
-        got = ops.flash_attention_with_fusing_bias_varlen(qp.to(gpu_device), kp.to(gpu_device), vp.to(gpu_device), dt,
+        dqp = dq.transpose(1, 2).reshape(B * L, H, D)
+        got = ops.flash_attention_with_fusing_bias_varlen(dqp, kp.to(gpu_device), vp.to(gpu_device), dt,
                                                           cu.to(gpu_device), cu.to(gpu_device), 512, 512,
                                                           sm_scale=1.0, exact_scores=exact)
         want = O.varlen_attention(qp, kp, vp, table, cu, cu, False, 1.0)

@@ -74,6 +74,87 @@ def test_attention_module_output_tuple(gpu_device):
             assert torch.isfinite(out[0][mask.bool()]).all()
 
 
+def test_output_attentions_gives_a_fourth_element_none(gpu_device):
+    """The reference's fused modules accept output_attentions=True and return None as the weights
+    (attentions.py:483, :519-520, :647, :860, :1063); so do these, with the other three elements unchanged."""
+    from turbot5_amd import T5ATTENTION_TYPES, T5Config
+    cfg = T5Config(**dict(SMALL, sliding_window=32, global_block_size=8))
+    x = torch.randn(2, 96, 128, device=gpu_device)
+    for name, cls in T5ATTENTION_TYPES.items():
+        mod = cls(cfg, has_relative_attention_bias=True).to(gpu_device).eval()
+        with torch.no_grad():
+            plain = mod(x)
+            out = mod(x, output_attentions=True)
+        assert len(plain) == 3 and len(out) == 4 and out[3] is None, name
+        assert torch.equal(out[0], plain[0]) and out[1] is None and out[2] is plain[2]
+
+
+@pytest.mark.parametrize("activations", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sigma", [8.0, 18.0])
+@pytest.mark.parametrize("kind", ["flash", "local", "block", "transient-global"])
+def test_modules_hold_2e2_at_unscaled_t5_score_magnitudes(gpu_device, kind, sigma, activations):
+    """T5 does not scale its scores, so trained checkpoints have scores of deviation 8 and more.  With the DEFAULT
+    config the modules fold log2(e) into the query projection (the rows are rounded to bf16 once, the kernel
+    applies no factor), and the attention output -- taken at the input of the output projection -- stays within
+    2e-2 of fp32 'basic' math on the rows, keys and values that the kernel was given: the rows divided by log2(e)
+    again, which costs a relative 2^-24.  fp32 activations with bf16 attention, and bf16 throughout."""
+    from turbot5_amd import T5ATTENTION_TYPES, T5Config, ops
+    from oracle import t5_basic as O
+    H, D, L, B, Bl, aux = 2, 64, 512, 2, 128, 16
+    cfg = T5Config(vocab_size=32, d_model=H * D, d_kv=D, d_ff=2 * H * D, num_layers=1, num_heads=H, dropout_rate=0.0,
+                   attention_type=kind, sliding_window=Bl, global_block_size=aux,
+                   attention_dtype=torch.bfloat16 if activations == torch.float32 else None)
+    assert cfg.attention_exact_scores is None
+    g = torch.Generator().manual_seed(int(sigma) * 7 + len(kind))
+    mod = T5ATTENTION_TYPES[kind](cfg, has_relative_attention_bias=True).eval()
+    with torch.no_grad():
+        # q.k over head_dim 64 has deviation sigma when the rows and keys have variance sigma / 8
+        std = (sigma / 8.0) ** 0.5
+        for name, prm in mod.named_parameters():
+            if "relative_attention_bias" in name:
+                prm.copy_(torch.randn(prm.shape, generator=g))
+            elif name.startswith(("q.", "k.")):
+                prm.copy_(torch.randn(prm.shape, generator=g) * std * prm.shape[1] ** -0.5)
+            elif name.startswith(("v.", "o.")):
+                prm.copy_(torch.randn(prm.shape, generator=g) * prm.shape[1] ** -0.5)
+    mod = mod.to(gpu_device).to(activations)
+    hidden = torch.randn(B, L, H * D, generator=g).to(gpu_device).to(activations)
+    seen = {}
+    mod.o.register_forward_pre_hook(lambda m, args: seen.__setitem__("attn", args[0].detach()))
+    calls = []
+    real = ops.prescaled_query
+    try:
+        ops.prescaled_query = lambda *a, **k: calls.append(real(*a, **k)) or calls[-1]
+        with torch.no_grad():
+            mod(hidden)
+    finally:
+        ops.prescaled_query = real
+    assert len(calls) == 1 and calls[0].dtype == torch.bfloat16   # the default config took the folded projection
+
+    def heads(x):
+        return x.float().cpu().view(B, -1, H, D).transpose(1, 2)
+    with torch.no_grad():
+        q = heads(calls[0]) / ops.LOG2E
+        k, v = (heads(p(hidden).to(torch.bfloat16)) for p in (mod.k, mod.v))
+        table = mod.relative_attention_bias.weight.float().cpu()
+        if kind == "flash":
+            want = O.dense_attention(q, k, v, table, False, 1.0)
+        elif kind == "local":
+            want = O.local_attention_blocked(q, k, v, table, Bl)
+        elif kind == "block":
+            want = O.block_attention_blocked(q, k, v, table, Bl, aux)
+        else:
+            side = mod.side_inputs(hidden)
+            sk, sv = (heads(p(side).to(torch.bfloat16)) for p in (mod.k, mod.v))
+            want = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, aux)
+    # the scores really are that large
+    s = torch.einsum("bhid,bhjd->bhij", q, k)
+    assert 0.8 * sigma <= s.std().item() <= 1.25 * sigma
+    got = heads(seen["attn"])
+    err = (got - want).abs().max().item()
+    assert err <= 2e-2, f"{kind} sigma {sigma}: max-abs {err}"
+
+
 def test_flash_encoder_with_padding(gpu_device):
     """A right-padded batch runs in place through the packed kernel with per-sequence lengths."""
     cfg, m, sd = make(dict(SMALL, attention_type="flash"))

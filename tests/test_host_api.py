@@ -35,7 +35,7 @@ def test_struct_sizes_follow_the_header(lib):
     assert C.sizeof(lib.T5ABias) == 8 + 4 * 4 + 2 * 8 + 2 * 8 + 2 * 4
     assert C.sizeof(lib.T5ADenseArgs) == 5 * 8 + 12 * 8 + 10 * 4 + C.sizeof(lib.T5ABias)
     assert C.sizeof(lib.T5AVarlenArgs) == 5 * 8 + 8 * 8 + 4 * 8 + 2 * 8 + 12 * 4 + C.sizeof(lib.T5ABias)
-    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 5 * 8
+    assert C.sizeof(lib.T5ASparseArgs) == 8 * 8 + 18 * 8 + 11 * 4 + 4 + C.sizeof(lib.T5ABias) + 5 * 8 + 2 * 4
     assert C.sizeof(lib.T5ASplitKArgs) == 7 * 8 + 16 * 8 + 8 * 4 + 2 * 8
     assert C.sizeof(lib.T5ARmsNormArgs) == 3 * 8 + 2 * 8 + 8 + 8 * 4 + 5 * 8 + 3 * 8
 
@@ -318,3 +318,47 @@ def test_packed_batch_layout_and_mask_kinds():
     _, (kind, (indices, cu, max_len), _) = A._mask_info(holes)
     assert kind == "packed" and indices.tolist() == [0, 2, 3, 5, 6, 7, 8, 9] and cu.tolist() == [0, 3, 8]
     assert A.packed_batch(holes).indices is indices
+
+
+@pytest.mark.parametrize("cus", [64, 104, 256, 304])
+def test_sparse_launch_plans_cover_every_item(lib, cus):
+    """The launch plan of the sparse patterns over a grid of shapes and device sizes: the runs cover the
+    (batch, head, q tile) list exactly, and when the global rows of the block pattern travel in the same launch,
+    their key splits cover the keys exactly, with at least one split per (batch, head) and never more than the
+    workspace was sized for.  Shapes with many (batch, head) pairs end with ONE split per pair: still a split item
+    of its own behind the runs (the kernel tells the folded launch by its number of block items)."""
+    L_ = lib.load()
+    out = (C.c_int32 * 6)()
+    seen_single_split = False
+    for B in (1, 2, 4, 8, 16, 33):
+        for H in (1, 8, 12, 16):
+            for L in (128, 500, 1024, 2048, 4096, 16384):
+                for Bl, G in ((128, 64), (64, 32), (256, 128), (100, 20), (512, 0)):
+                    if G > Bl:
+                        continue
+                    for run_len in (0, 1, 5, 16):
+                        rc = L_.t5a_sparse_launch_plan(lib.PATTERN_BLOCK, lib.T5A_BF16, B, H, L, 64, Bl, G, 1, cus, run_len, out)
+                        assert rc == 0, (B, H, L, Bl, G, run_len, L_.t5a_last_error())
+                        rl, items, block_items, nsplit, split_rows, tps = list(out)
+                        entries = tps * B * H
+                        runs = block_items if block_items > 0 else items
+                        assert 1 <= rl <= 16 and runs * rl >= entries > (runs - 1) * rl, (B, H, L, Bl, G, run_len, list(out))
+                        if run_len:
+                            assert rl == run_len or L < Bl
+                        if block_items > 0:
+                            assert items == block_items + nsplit * B * H and nsplit >= 1
+                            assert nsplit * split_rows >= L > (nsplit - 1) * split_rows and split_rows % 64 == 0
+                            ws = L_.t5a_sparse_workspace_bytes(lib.PATTERN_BLOCK, B, H, L, 64, Bl, G)
+                            assert B * H * nsplit * min(G, L) * (64 + 2) * 4 <= ws
+                            seen_single_split |= nsplit == 1
+                        else:
+                            assert nsplit == 0
+    assert seen_single_split or cus > 256
+    # the local pattern: runs only; fp32 and other head dims: one q tile per item
+    for dtype, D, want_runs in ((lib.T5A_BF16, 64, True), (lib.T5A_F32, 64, False), (lib.T5A_BF16, 32, False)):
+        assert L_.t5a_sparse_launch_plan(lib.PATTERN_LOCAL, dtype, 1, 12, 16384, D, 128, 0, 0, cus, 0, out) == 0
+        rl, items, block_items, nsplit, split_rows, tps = list(out)
+        assert tps == 128 and block_items == 0 and items * rl >= 128 * 12 > (items - 1) * rl
+        assert (rl > 1) == (want_runs and 2 * cus < 128 * 12)
+    assert L_.t5a_sparse_launch_plan(lib.PATTERN_BLOCK, lib.T5A_BF16, 1, 1, 128, 64, 128, 64, 1, cus, 17, out) < 0
+    assert L_.t5a_sparse_launch_plan(9, lib.T5A_BF16, 1, 1, 128, 64, 128, 64, 1, cus, 0, out) < 0

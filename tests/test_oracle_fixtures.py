@@ -34,20 +34,27 @@ def heads(x, H, D):
     return x.view(B, L, H, D).transpose(1, 2)
 
 
-def oracle_module_output(name, c):
-    """The module's forward restated with the oracle's op-level functions."""
+def oracle_attention_output(name, c):
+    """The module's attention op restated with the oracle's op-level functions: (B, H, L, D), head-correct, before
+    the head merge and the output projection."""
     B, L, H, D, Bl, aux = (int(x) for x in c["meta"])
     hidden, mask = c["hidden"], c["mask"]
     q, k, v = (heads(hidden @ c[f"w.{n}.weight"].T, H, D) for n in ("q", "k", "v"))
     table = c["w.relative_attention_bias.weight"]
     if "Block" in name:
-        o = O.block_attention_blocked(q, k, v, table, Bl, aux, mask)
-    elif "Local" in name:
-        o = O.local_attention_blocked(q, k, v, table, Bl, mask)
-    else:
-        side = O.tglobal_side_inputs(hidden, mask, aux, c["w.global_input_layer_norm.weight"])
-        sk, sv = (heads(side @ c[f"w.{n}.weight"].T, H, D) for n in ("k", "v"))
-        o = O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, aux, mask)
+        return O.block_attention_blocked(q, k, v, table, Bl, aux, mask)
+    if "Local" in name:
+        return O.local_attention_blocked(q, k, v, table, Bl, mask)
+    side = O.tglobal_side_inputs(hidden, mask, aux, c["w.global_input_layer_norm.weight"])
+    sk, sv = (heads(side @ c[f"w.{n}.weight"].T, H, D) for n in ("k", "v"))
+    return O.tglobal_attention_blocked(q, k, v, sk, sv, table, Bl, aux, mask)
+
+
+def oracle_module_output(name, c):
+    """The module's forward: the attention op above, the module's head merge and its output projection."""
+    B, L, H, D, Bl, aux = (int(x) for x in c["meta"])
+    o = oracle_attention_output(name, c)
+    if "TransientGlobal" in name:
         # the reference module merges heads without the head transpose (attentions.py:951-953): its rows are
         # the (block, head, row-in-block) order read as (row, head).  Reproduce that here, outside the op.
         nb = -(-L // Bl) if L >= Bl else 1

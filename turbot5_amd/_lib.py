@@ -13,14 +13,15 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 112   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 113   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
+SCORES_DEFAULT, SCORES_EXACT, SCORES_PRESCALED = 0, 1, 2   # the exact_scores field
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_fwd_varlen",
     "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes", "t5a_bias_lut_bytes_windowed",
-    "t5a_fwd_sparse", "t5a_sparse_workspace_bytes", "t5a_sparse_key_bits_words", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
+    "t5a_fwd_sparse", "t5a_sparse_launch_plan", "t5a_sparse_workspace_bytes", "t5a_sparse_key_bits_words", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
     "t5a_rmsnorm",
 )
 
@@ -67,7 +68,8 @@ class T5ASparseArgs(C.Structure):
                 ("pattern", C.c_int32), ("block_len", C.c_int32), ("aux", C.c_int32), ("n_side", C.c_int32),
                 ("sm_scale", C.c_float), ("exact_scores", C.c_int32),
                 ("bias", T5ABias), ("seq_lens", C.c_void_p), ("seq_starts", C.c_void_p),
-                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64), ("side_counts", C.c_void_p)]
+                ("key_bits", C.c_void_p), ("key_bits_stride", C.c_int64), ("side_counts", C.c_void_p),
+                ("run_len", C.c_int32), ("reserved", C.c_int32)]
 
 
 class T5ASplitKArgs(C.Structure):
@@ -139,6 +141,8 @@ def load() -> C.CDLL:
         lib.t5a_varlen_workspace_bytes.restype = C.c_int64
         lib.t5a_sparse_workspace_bytes.argtypes = [C.c_int32] * 7
         lib.t5a_sparse_workspace_bytes.restype = C.c_int64
+        lib.t5a_sparse_launch_plan.argtypes = [C.c_int32] * 11 + [C.POINTER(C.c_int32)]
+        lib.t5a_sparse_launch_plan.restype = C.c_int
         lib.t5a_sparse_key_bits_words.argtypes = [C.c_int32] * 3
         lib.t5a_sparse_key_bits_words.restype = C.c_int64
         _lib = lib

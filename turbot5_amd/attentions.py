@@ -17,7 +17,8 @@ Differences from the reference, all on purpose:
   and for local / transient-global also left padding); masks with holes raise ``NotImplementedError``;
 * transient-global returns the head-correct layout (the reference's ``unshape`` omits the
   head transpose, attentions.py:951-953);
-* ``layer_head_mask`` and ``output_attentions`` are not available on fused paths.
+* ``layer_head_mask`` is not available on fused paths; ``output_attentions=True`` adds a fourth element None to the
+  returned tuple, as the reference's fused modules do (attentions.py:483, :519-520, :647, :860, :1063).
 """
 from __future__ import annotations
 
@@ -181,10 +182,18 @@ class _T5AttentionBase(nn.Module):
     def _attn_dtype(self, x: torch.Tensor) -> torch.dtype:
         return self.config.attention_dtype or x.dtype
 
-    @property
-    def _exact(self):
-        """None (library default) or the config's choice of score precision, see ``ops.EXACT_SCORES``."""
-        return getattr(self.config, "attention_exact_scores", None)
+    def _query(self, hidden_states: torch.Tensor, adt: torch.dtype):
+        """-> (query rows (..., H*D) in the attention dtype, the ``exact_scores`` argument that goes with them).
+
+        16-bit attention, ``config.attention_exact_scores`` None: log2(e) is folded into the projection
+        (``ops.prescaled_query``), so the rows are rounded to the attention dtype once and the kernel applies no
+        factor to them -- the reference applies its factor to the fp32 product (fused_bias_attention.py:323-337);
+        this gives the same accuracy without the multiply per score.  True / False: plain projection, the
+        kernel scales the fp32 product / multiplies and re-rounds the rows."""
+        choice = getattr(self.config, "attention_exact_scores", None)
+        if choice is None and adt in (torch.bfloat16, torch.float16) and hidden_states.is_cuda:
+            return ops.prescaled_query(hidden_states, self.q.weight, adt, 1.0), "prescaled"
+        return self.q(hidden_states).to(adt), choice
 
     def _table(self, position_bias):
         if position_bias is None and self.has_relative_attention_bias:
@@ -196,10 +205,15 @@ class _T5AttentionBase(nn.Module):
 
     @staticmethod
     def _reject(layer_head_mask, output_attentions):
+        """``output_attentions=True`` is accepted as in the reference's fused modules, whose fourth tuple element is
+        then None (attentions.py:483, :519-520, :647, :860, :1063): the weights are never materialised."""
         if layer_head_mask is not None:
             raise NotImplementedError("layer_head_mask is not supported by the fused attention kernels")
-        if output_attentions:
-            raise NotImplementedError("attention weights are never materialised by the fused attention kernels")
+
+    @staticmethod
+    def _outputs(attn_output, present_key_value, table, output_attentions):
+        outputs = (attn_output, present_key_value, table)
+        return outputs + (None,) if output_attentions else outputs
 
 
 class T5FlashAttention(_T5AttentionBase):
@@ -254,7 +268,10 @@ class T5FlashAttention(_T5AttentionBase):
                 return self._shape(proj_layer(key_value_states), batch_size).to(adt)
             return past
 
-        query_states = self._shape(self.q(hidden_states), batch_size).to(adt)
+        query_rows, exact = self._query(hidden_states, adt)
+        query_states = self._shape(query_rows, batch_size)
+        # (the split-K kernel scales the fp32 product: rows that carry log2(e) already get ln 2 as their scale)
+        dec_scale = 1.0 / ops.LOG2E if exact == "prescaled" else 1.0
         key_states = project(self.k, past_key_value[0] if past_key_value is not None else None)
         value_states = project(self.v, past_key_value[1] if past_key_value is not None else None)
         table = self._table(position_bias)
@@ -264,10 +281,10 @@ class T5FlashAttention(_T5AttentionBase):
         if not varlen:
             if table is None and not self.causal and seq_length <= 8 and key_length >= 512:
                 # few query rows over a long memory (incremental decoding): split-K kernel
-                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, 1.0)
+                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, dec_scale)
             else:
                 attn_output = ops.flash_attention_with_fusing_bias(
-                    query_states, key_states, value_states, table, causal=self.causal, sm_scale=1.0, exact_scores=self._exact,
+                    query_states, key_states, value_states, table, causal=self.causal, sm_scale=1.0, exact_scores=exact,
                     NUM_BUCKETS=nb, MAX_DISTANCE=md)
         else:
             if mask.shape[1] != key_length:
@@ -291,7 +308,7 @@ class T5FlashAttention(_T5AttentionBase):
                 if starts is None:
                     starts = plans["key_starts"] = (cu_k[:batch_size] - torch.arange(
                         batch_size, device=dev, dtype=torch.int32) * key_length).contiguous()
-                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, 1.0,
+                attn_output = ops.flash_decoding_attention(query_states, key_states, value_states, None, dec_scale,
                                                            key_lens=lens_k, key_starts=starts)
                 kind = "done"
             elif kind == "lens":
@@ -306,7 +323,7 @@ class T5FlashAttention(_T5AttentionBase):
                                                            dtype=torch.int32, device=dev)
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
                     rows(q_blhd, seq_length), rows(k_blhd, key_length), rows(v_blhd, key_length), table, cu_q, cu_k,
-                    seq_length, key_length, causal=self.causal, sm_scale=1.0, exact_scores=self._exact, NUM_BUCKETS=nb, MAX_DISTANCE=md,
+                    seq_length, key_length, causal=self.causal, sm_scale=1.0, exact_scores=exact, NUM_BUCKETS=nb, MAX_DISTANCE=md,
                     seq_lens_q=unpad if self_attn else None, seq_lens_k=unpad,
                     launch_plan=plan)
                 attn_output = out_p.view(batch_size, seq_length, self.n_heads, -1).transpose(1, 2)
@@ -324,7 +341,7 @@ class T5FlashAttention(_T5AttentionBase):
                 indices_q, max_q = None, seq_length
             if kind not in ("lens", "done"):
                 out_p = ops.flash_attention_with_fusing_bias_varlen(
-                    q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0, exact_scores=self._exact,
+                    q_p, k_p, v_p, table, cu_q, cu_k, max_q, max_k, causal=self.causal, sm_scale=1.0, exact_scores=exact,
                     NUM_BUCKETS=nb, MAX_DISTANCE=md, launch_plan=plan)
                 if indices_q is not None:
                     attn_output = pad_input(out_p, indices_q, batch_size, seq_length).transpose(1, 2)
@@ -333,7 +350,7 @@ class T5FlashAttention(_T5AttentionBase):
 
         attn_output = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
         present_key_value_state = (key_states, value_states) if (self.is_decoder and use_cache) else None
-        return (attn_output,) + (present_key_value_state,) + (table,)
+        return self._outputs(attn_output, present_key_value_state, table, output_attentions)
 
     def forward_packed(self, hidden_states, packed: PackedBatch, position_bias=None):
         """Self-attention over hidden states that are already packed: (total, d_model), sequences back to
@@ -341,14 +358,15 @@ class T5FlashAttention(_T5AttentionBase):
         sequence, as in the reference's packed call (varlen_fused_bias_attn.py:254, :303)."""
         total = hidden_states.shape[0]
         adt = self._attn_dtype(hidden_states)
-        q, k, v = (p(hidden_states).view(total, self.n_heads, self.key_value_proj_dim).to(adt)
-                   for p in (self.q, self.k, self.v))
+        q, exact = self._query(hidden_states, adt)
+        q = q.view(total, self.n_heads, self.key_value_proj_dim)
+        k, v = (p(hidden_states).view(total, self.n_heads, self.key_value_proj_dim).to(adt) for p in (self.k, self.v))
         table = self._table(position_bias)
         plan = packed.plans.setdefault((self.causal, self.n_heads, self.key_value_proj_dim, adt,
                                         ops._stream(hidden_states)), ops.LaunchPlan())
         out = ops.flash_attention_with_fusing_bias_varlen(
             q, k, v, table, packed.cu_seqlens, packed.cu_seqlens, packed.max_len, packed.max_len,
-            causal=self.causal, sm_scale=1.0, exact_scores=self._exact, NUM_BUCKETS=self.relative_attention_num_buckets,
+            causal=self.causal, sm_scale=1.0, exact_scores=exact, NUM_BUCKETS=self.relative_attention_num_buckets,
             MAX_DISTANCE=self.relative_attention_max_distance, launch_plan=plan)
         return (self.o(out.reshape(total, self.inner_dim).to(hidden_states.dtype)), None, table)
 
@@ -392,14 +410,17 @@ class _SparseBase(_T5AttentionBase):
         return None, None
 
     def _qkv(self, hidden_states):
+        """-> q, k, v as (B, H, L, D) views in the attention dtype and the ``exact_scores`` argument for q"""
         batch_size = hidden_states.shape[0]
         adt = self._attn_dtype(hidden_states)
-        return tuple(self._shape(p(hidden_states), batch_size).to(adt) for p in (self.q, self.k, self.v))
+        q, exact = self._query(hidden_states, adt)
+        k, v = (self._shape(p(hidden_states), batch_size).to(adt) for p in (self.k, self.v))
+        return self._shape(q, batch_size), k, v, exact
 
-    def _finish(self, attn_output, hidden_states, table):
+    def _finish(self, attn_output, hidden_states, table, output_attentions=False):
         batch_size = hidden_states.shape[0]
         out = self.o(self._unshape(attn_output, batch_size).to(hidden_states.dtype))
-        return (out,) + (None,) + (table,)
+        return self._outputs(out, None, table, output_attentions)
 
 
 class T5LocalAttention(_SparseBase):
@@ -414,7 +435,7 @@ class T5LocalAttention(_SparseBase):
         # right-padded batches: the keys of a sequence end at its length (the key half of the reference's
         # local mask, utils.py:174-188); outputs at padded positions mean nothing, as in the reference
         seq_lens, seq_starts = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions)
-        q, k, v = self._qkv(hidden_states)
+        q, k, v, exact = self._qkv(hidden_states)
         table = self._table(position_bias)
         # a sequence shorter than one block is a single block of its own length (utils.py:107-108)
         block_len = min(self.block_len, hidden_states.shape[1])
@@ -424,8 +445,8 @@ class T5LocalAttention(_SparseBase):
         out = ops.local_attention_with_fusing_bias(
             q, k, v, table, block_len, 1.0, self.relative_attention_num_buckets,
             self.relative_attention_max_distance, seq_lens=seq_lens, seq_starts=seq_starts,
-            exact_scores=self._exact, key_bits=key_bits)
-        return self._finish(out, hidden_states, table)
+            exact_scores=exact, key_bits=key_bits)
+        return self._finish(out, hidden_states, table, output_attentions)
 
 
 class T5BlockAttention(_SparseBase):
@@ -442,17 +463,27 @@ class T5BlockAttention(_SparseBase):
         # (left padding and holes: validity bit sets, looked up per tile)
         seq_lens, _ = self._check_call(mask, layer_head_mask, past_key_value, use_cache, output_attentions,
                                        left_padding_ok=False)
-        if seq_lens is not None and hidden_states.shape[1] < self.block_len:
-            raise NotImplementedError("T5BlockAttention: padded batches shorter than one block are not supported")
-        q, k, v = self._qkv(hidden_states)
+        q, k, v, exact = self._qkv(hidden_states)
         table = self._table(position_bias)
         key_bits = None
+        seq_length = hidden_states.shape[1]
+        if seq_lens is not None and seq_length < self.block_len:
+            # A padded batch shorter than one block: the reference's single block of seq_length keys under the
+            # additive key mask, bias of the row distance (attentions.py:752, :691, :722-732) -- full attention
+            # over the valid keys with positions = row indices, which is the windowed kernel with a window that
+            # spans the sequence.
+            if isinstance(seq_lens, str):
+                seq_lens, key_bits = None, self._key_bits(mask, seq_length)
+            out = ops.local_attention_with_fusing_bias(
+                q, k, v, table, seq_length, 1.0, self.relative_attention_num_buckets,
+                self.relative_attention_max_distance, seq_lens=seq_lens, exact_scores=exact, key_bits=key_bits)
+            return self._finish(out, hidden_states, table, output_attentions)
         if isinstance(seq_lens, str):
             seq_lens, key_bits = None, self._key_bits(mask, self.block_len, self.n_global_tokens)
         out = ops.block_attention_with_fusing_bias(
             q, k, v, table, self.block_len, self.n_global_tokens, 1.0, self.relative_attention_num_buckets,
-            self.relative_attention_max_distance, exact_scores=self._exact, seq_lens=seq_lens, key_bits=key_bits)
-        return self._finish(out, hidden_states, table)
+            self.relative_attention_max_distance, exact_scores=exact, seq_lens=seq_lens, key_bits=key_bits)
+        return self._finish(out, hidden_states, table, output_attentions)
 
 
 class T5TransientGlobalAttention(_SparseBase):
@@ -498,7 +529,7 @@ class T5TransientGlobalAttention(_SparseBase):
             side_counts = plans.get(("side_counts", self.global_block_size))
             if side_counts is None:
                 side_counts = plans[("side_counts", self.global_block_size)] = ops.side_token_counts(mask, self.global_block_size)
-        q, k, v = self._qkv(hidden_states)
+        q, k, v, exact = self._qkv(hidden_states)
         side = self.side_inputs(hidden_states, seq_lens, seq_starts, key_bits, side_counts)
         side_k = self._shape(self.k(side), batch_size).to(adt)
         side_v = self._shape(self.v(side), batch_size).to(adt)
@@ -506,8 +537,8 @@ class T5TransientGlobalAttention(_SparseBase):
         out = ops.transient_global_attention_with_fusing_bias(
             q, k, v, side_k, side_v, table, block_len, self.global_block_size, 1.0,
             self.relative_attention_num_buckets, self.relative_attention_max_distance, seq_lens=seq_lens,
-            seq_starts=seq_starts, exact_scores=self._exact, key_bits=key_bits, side_counts=side_counts)
-        return self._finish(out, hidden_states, table)
+            seq_starts=seq_starts, exact_scores=exact, key_bits=key_bits, side_counts=side_counts)
+        return self._finish(out, hidden_states, table, output_attentions)
 
 
 T5ATTENTION_TYPES = {

@@ -72,20 +72,5 @@ def build(verbose: bool = False, jobs: int = 8, extra_flags=(), trace: bool = Fa
     return lib
 
 
-MEASURE_SRC = os.path.join(CSRC, "measure", "issue_costs.hip")
-MEASURE_BIN = os.path.join(CSRC, "measure", "issue_costs")
-
-
-def build_measure(verbose: bool = False) -> str:
-    """The instruction-cost microbenchmarks behind the design notes (a stand-alone executable, not part of the
-    library): cycles per instruction of the tile loop's instruction mix, LDS read throughput."""
-    _run([_hipcc(), "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-Wno-unused-result", MEASURE_SRC, "-o", MEASURE_BIN],
-         verbose)
-    return MEASURE_BIN
-
-
 if __name__ == "__main__":
-    if "--measure" in sys.argv:
-        print(build_measure(verbose="-v" in sys.argv))
-    else:
-        print(build(verbose="-v" in sys.argv, trace="--trace" in sys.argv))
+    print(build(verbose="-v" in sys.argv, trace="--trace" in sys.argv))

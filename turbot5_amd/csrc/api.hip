@@ -171,6 +171,19 @@ static int finish(hipError_t e, const char* what) {
 
 static const float kLog2e = 1.4426950408889634f;
 
+// How sm_scale * log2(e) reaches the scores (the exact_scores field of the argument structs).
+//   T5A_SCORES_DEFAULT   16-bit inputs: Q is multiplied by the factor in the kernel and rounded back to its type
+//   T5A_SCORES_EXACT     the factor is applied to the fp32 product (fused_bias_attention.py:323-337 does this)
+//   T5A_SCORES_PRESCALED the caller's Q already carries sm_scale * log2(e) (folded into the projection that made
+//                        it, so that Q was rounded to its type once): the kernel multiplies by exactly 1
+static int score_mode(int mode, float sm_scale, FwdParams* p) {
+    if (mode != T5A_SCORES_DEFAULT && mode != T5A_SCORES_EXACT && mode != T5A_SCORES_PRESCALED)
+        return fail(T5A_ERR_SHAPE, "exact_scores=%d is none of T5A_SCORES_DEFAULT, _EXACT, _PRESCALED", mode);
+    p->c1 = mode == T5A_SCORES_PRESCALED ? 1.0f : sm_scale * kLog2e;
+    p->exact_scale = mode == T5A_SCORES_EXACT;
+    return T5A_OK;
+}
+
 static hipError_t launch_fwd(const FwdParams& p, int dtype, int D, int mode, bool causal, hipStream_t stream) {
     if (p.total_items <= 0) return hipSuccess;
     if (dtype == T5A_BF16) return launch_fwd_bf16(p, D, mode, causal, stream);
@@ -270,8 +283,7 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     if (items > 0x7fffff00LL) return fail(T5A_ERR_SHAPE, "too many work items (%lld)", (long long)items);
     p.total_items = (int)items;
     if (a->causal != 0 && p.tiles_per_seq > 1) causal_slices(&p, a->dtype, a->D);
-    p.c1 = a->sm_scale * kLog2e;
-    p.exact_scale = a->exact_scores != 0;
+    if ((rc = score_mode(a->exact_scores, a->sm_scale, &p))) return rc;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
     if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
@@ -323,8 +335,7 @@ int t5a_fwd_varlen(const t5a_varlen_args* a, t5a_stream_t stream) {
     p.total_items = (int)items;
     p.tiles_per_seq = 1;
     p.align_end = 1;
-    p.c1 = a->sm_scale * kLog2e;
-    p.exact_scale = a->exact_scores != 0;
+    if ((rc = score_mode(a->exact_scores, a->sm_scale, &p))) return rc;
     if ((rc = fill_bias(a->bias, a->causal == 0, &p))) return rc;
     if ((rc = prepare_lut(a->bias, a->causal != 0, (hipStream_t)stream, &p))) return rc;
     const int64_t need = t5a_varlen_workspace_bytes(a->B, a->H, a->total_q);
@@ -378,7 +389,7 @@ static int device_compute_units() {
 // pattern is only a few steps long, about as long as the set-up of a work item, which a run pays once; longer runs
 // mean fewer workgroups.  Two workgroups fit a compute unit: count the rounds the device needs for the runs and
 // charge every round its q tiles plus one set-up.
-static void choose_runs(FwdParams* p, int mode, int dtype, int D, int64_t other_items = 0) {
+static void choose_runs(FwdParams* p, int mode, int dtype, int D, int cus, int forced_run_len, int64_t other_items = 0) {
     p->run_len = 1;
     p->runs_per_seq = p->tiles_per_seq;
     const int64_t entries = (int64_t)p->tiles_per_seq * p->H * p->B;   // the (batch, head, q tile) list
@@ -387,17 +398,13 @@ static void choose_runs(FwdParams* p, int mode, int dtype, int D, int64_t other_
     if (runs_ok) {
         // as many workgroups as the device holds at once (two per compute unit), each with its share of the list;
         // other_items: workgroups of the same launch that are not runs (the block pattern's key splits)
-        int64_t slots = 2 * (int64_t)device_compute_units() - other_items;
+        int64_t slots = 2 * (int64_t)cus - other_items;
         if (slots < 64) slots = 64;
         int64_t rl = (entries + slots - 1) / slots;
-        if (rl > 16) rl = 16;
+        if (rl > kMaxRunLen) rl = kMaxRunLen;
         if (rl < 1) rl = 1;
         p->run_len = (int)rl;
-        // T5A_RUN_LEN=<n>: fixed run length, for tests and measurements
-        if (const char* e = getenv("T5A_RUN_LEN")) {
-            const int forced = atoi(e);
-            if (forced >= 1) p->run_len = forced;
-        }
+        if (forced_run_len >= 1) p->run_len = forced_run_len;   // the caller's choice (validated: 1 .. kMaxRunLen)
     }
     p->total_items = (int)((entries + p->run_len - 1) / p->run_len);
 }
@@ -420,33 +427,34 @@ static void global_row_splits(int B, int H, int L, int* nsplit, int* split_rows)
 // Costs in thousands of cycles, measured on an MI355X: a run pays one set-up (15) and per q tile three steps and
 // the switch to the next q tile (15.6); a split pays one set-up (16) and 2.0 per key tile.  Never more splits than
 // global_row_splits() gives: the workspace size is computed from that.
-static void block_fold_plan(FwdParams* p, int dtype, int D, int B, int H, int L, int* nsplit, int* split_rows) {
+static void block_fold_plan(FwdParams* p, int dtype, int D, int B, int H, int L, int cus, int forced_run_len,
+                            int* nsplit, int* split_rows) {
     global_row_splits(B, H, L, nsplit, split_rows);
+    const int most_splits = *nsplit;   // what the workspace was sized for
     const int64_t bh = (int64_t)B * H;
     const int64_t entries = (int64_t)p->tiles_per_seq * bh;
-    const int64_t slots = 2 * (int64_t)device_compute_units();
+    const int64_t slots = 2 * (int64_t)cus;
     const bool runs_ok = dtype != T5A_F32 && (D == 64 || D == 128);
-    if (!runs_ok || getenv("T5A_RUN_LEN") != nullptr || entries + (int64_t)*nsplit * bh <= slots) {
-        choose_runs(p, kBlock, dtype, D, (int64_t)*nsplit * bh);
+    if (!runs_ok || forced_run_len >= 1 || entries + (int64_t)*nsplit * bh <= slots) {
+        choose_runs(p, kBlock, dtype, D, cus, forced_run_len, (int64_t)*nsplit * bh);
         return;
     }
     const int tiles = (L + 63) / 64;
     double best = 0.0;
     int best_r = 0, best_s = 0;
-    for (int r = 1; r <= 16; ++r) {
+    for (int r = 1; r <= kMaxRunLen; ++r) {
         const int64_t n_runs = (entries + r - 1) / r;
         const int64_t free_slots = slots - n_runs;
         if (free_slots < bh) continue;
-        int64_t per_bh = free_slots / bh;
-        if (per_bh > *nsplit) per_bh = *nsplit;
-        if (per_bh < 1) per_bh = 1;
+        int64_t per_bh = free_slots / bh;   // >= 1: one split is a whole pass over the keys, still an item of its own
+        if (per_bh > most_splits) per_bh = most_splits;
         const int s_tiles = (int)((tiles + per_bh - 1) / per_bh);
         const double run_cost = 15.0 + 15.6 * r, split_cost = 16.0 + 2.0 * s_tiles;
         const double cost = run_cost > split_cost ? run_cost : split_cost;
         if (best_r == 0 || cost < best) { best = cost; best_r = r; best_s = s_tiles; }
     }
     if (best_r == 0) {   // more work than one round holds at any run length
-        choose_runs(p, kBlock, dtype, D, (int64_t)*nsplit * bh);
+        choose_runs(p, kBlock, dtype, D, cus, forced_run_len, (int64_t)*nsplit * bh);
         return;
     }
     p->run_len = best_r;
@@ -454,6 +462,24 @@ static void block_fold_plan(FwdParams* p, int dtype, int D, int B, int H, int L,
     p->total_items = (int)((entries + best_r - 1) / best_r);
     *split_rows = best_s * 64;
     *nsplit = (tiles + best_s - 1) / best_s;
+}
+
+// What a folded block launch must satisfy before it may start (every item index the kernel decodes stays inside
+// the lists): the runs cover the (batch, head, q tile) list, the splits cover the keys, and there are no more
+// splits than the workspace holds.
+static int check_fold_plan(const FwdParams& p, int B, int H, int L, int nsplit, int split_rows) {
+    int most, rows_unused;
+    global_row_splits(B, H, L, &most, &rows_unused);
+    const int64_t entries = (int64_t)p.tiles_per_seq * H * B;
+    if (p.run_len < 1 || p.run_len > kMaxRunLen || (int64_t)p.total_items * p.run_len < entries ||
+        (int64_t)(p.total_items - 1) * p.run_len >= entries)
+        return fail(T5A_ERR_LAUNCH, "block launch plan: %d runs of %d q tiles do not cover %lld entries", p.total_items,
+                    p.run_len, (long long)entries);
+    if (nsplit < 1 || nsplit > most || split_rows < 64 || split_rows % 64 != 0 || (int64_t)nsplit * split_rows < L ||
+        (int64_t)(nsplit - 1) * split_rows >= L)
+        return fail(T5A_ERR_LAUNCH, "block launch plan: %d key splits of %d rows do not cover %d keys (at most %d splits)",
+                    nsplit, split_rows, L, most);
+    return T5A_OK;
 }
 
 int64_t t5a_sparse_key_bits_words(int32_t L, int32_t block_len, int32_t aux) {
@@ -472,6 +498,45 @@ int64_t t5a_sparse_workspace_bytes(int32_t pattern, int32_t B, int32_t H, int32_
     return (int64_t)B * H * nsplit * G * ((int64_t)D + 2) * (int64_t)sizeof(float);
 }
 
+int t5a_sparse_launch_plan(int32_t pattern, int32_t dtype, int32_t B, int32_t H, int32_t L, int32_t D, int32_t block_len,
+                           int32_t aux, int32_t with_workspace, int32_t compute_units, int32_t run_len, int32_t* out) {
+    if (out == nullptr) return fail(T5A_ERR_NULL, "out is NULL");
+    int rc = check_common(dtype, D);
+    if (rc) return rc;
+    if (B <= 0 || H <= 0 || L <= 0 || block_len <= 0 || aux < 0 || run_len < 0 || run_len > kMaxRunLen)
+        return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d L=%d block_len=%d aux=%d run_len=%d", B, H, L, block_len, aux, run_len);
+    const int cus = compute_units > 0 ? compute_units : device_compute_units();
+    FwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.B = B; p.H = H; p.M = L; p.N = L;
+    int nsplit = 0, split_rows = 0, block_items = 0;
+    if (pattern == T5A_PATTERN_BLOCK && L >= block_len) {
+        p.tiles_per_seq = ((L + block_len - 1) / block_len) * ((block_len + 127) / 128);
+        const int G = aux < L ? aux : L;
+        const bool fold = aux > 0 && with_workspace != 0 && G <= 128 &&
+                          t5a_sparse_workspace_bytes(pattern, B, H, L, D, block_len, aux) > 0;
+        if (fold) {
+            block_fold_plan(&p, dtype, D, B, H, L, cus, run_len, &nsplit, &split_rows);
+            if ((rc = check_fold_plan(p, B, H, L, nsplit, split_rows))) return rc;
+            block_items = p.total_items;
+            p.total_items += nsplit * H * B;
+        } else {
+            choose_runs(&p, kBlock, dtype, D, cus, run_len);
+        }
+    } else if (pattern == T5A_PATTERN_LOCAL || pattern == T5A_PATTERN_TGLOBAL || pattern == T5A_PATTERN_BLOCK) {
+        // (a block pattern over less than one block runs as full attention)
+        p.tiles_per_seq = (L + 127) / 128;
+        const int mode = pattern == T5A_PATTERN_BLOCK ? kDense : pattern == T5A_PATTERN_TGLOBAL ? kTGlobal
+                         : (block_len <= kMaxLutWindow ? kLocal : kLocalWide);
+        choose_runs(&p, mode, dtype, D, cus, run_len);
+    } else {
+        return fail(T5A_ERR_PATTERN, "unknown pattern %d", pattern);
+    }
+    out[0] = p.run_len; out[1] = p.total_items; out[2] = block_items; out[3] = nsplit; out[4] = split_rows;
+    out[5] = p.tiles_per_seq;
+    return T5A_OK;
+}
+
 int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
@@ -485,7 +550,10 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         return fail(T5A_ERR_PATTERN, "block pattern needs 0 <= n_global (%d) <= block_len (%d)", a->aux, a->block_len);
     if (a->pattern == T5A_PATTERN_TGLOBAL && (a->aux <= 0 || a->n_side < 0))
         return fail(T5A_ERR_PATTERN, "transient-global needs aux > 0 and n_side >= 0 (aux=%d n_side=%d)", a->aux, a->n_side);
+    if (a->run_len < 0 || a->run_len > kMaxRunLen)
+        return fail(T5A_ERR_SHAPE, "run_len=%d: 0 (the library chooses) or 1..%d", a->run_len, kMaxRunLen);
     if (a->B == 0 || a->L == 0) return T5A_OK;
+    const int cus = device_compute_units();
     if ((rc = check_tensor("q", a->q, a->q_strides, 3, unit))) return rc;
     if ((rc = check_tensor("k", a->k, a->k_strides, 3, unit))) return rc;
     if ((rc = check_tensor("v", a->v, a->v_strides, 3, unit))) return rc;
@@ -530,8 +598,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         if (a->pattern == T5A_PATTERN_TGLOBAL) p.side_counts = a->side_counts;
     }
     p.block_len = a->block_len; p.aux = a->aux; p.n_side = a->n_side;
-    p.c1 = a->sm_scale * kLog2e;
-    p.exact_scale = a->exact_scores != 0;
+    if ((rc = score_mode(a->exact_scores, a->sm_scale, &p))) return rc;
     if ((rc = fill_bias(a->bias, true, &p))) return rc;
     hipStream_t s = (hipStream_t)stream;
     const bool window_in_lut = a->pattern == T5A_PATTERN_LOCAL && a->block_len <= kMaxLutWindow && a->key_bits == nullptr;
@@ -554,9 +621,10 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
         const int64_t need = t5a_sparse_workspace_bytes(a->pattern, a->B, a->H, a->L, a->D, a->block_len, a->aux);
         const bool fold = a->aux > 0 && a->workspace != nullptr && need > 0 && G <= 128;
         int fold_splits = 0, fold_rows = 0;
-        if (fold) block_fold_plan(&p, a->dtype, a->D, a->B, a->H, a->L, &fold_splits, &fold_rows);
-        else choose_runs(&p, kBlock, a->dtype, a->D);
+        if (fold) block_fold_plan(&p, a->dtype, a->D, a->B, a->H, a->L, cus, a->run_len, &fold_splits, &fold_rows);
+        else choose_runs(&p, kBlock, a->dtype, a->D, cus, a->run_len);
         if (fold) {
+            if ((rc = check_fold_plan(p, a->B, a->H, a->L, fold_splits, fold_rows))) return rc;
             // one launch: the block items, then the global rows as key splits spread over the whole device; one merge
             if (a->workspace_bytes < need)
                 return fail(T5A_ERR_WORKSPACE, "workspace of %lld bytes, %lld needed", (long long)a->workspace_bytes, (long long)need);
@@ -619,7 +687,7 @@ int t5a_fwd_sparse(const t5a_sparse_args* a, t5a_stream_t stream) {
     // (validity bit sets go with the instantiation that masks per element)
     const int mode = a->pattern == T5A_PATTERN_TGLOBAL ? (a->key_bits != nullptr ? kTGlobalBits : kTGlobal)
                      : (a->block_len <= kMaxLutWindow && a->key_bits == nullptr ? kLocal : kLocalWide);
-    choose_runs(&p, mode, a->dtype, a->D);
+    choose_runs(&p, mode, a->dtype, a->D, cus, a->run_len);
     return finish(launch_fwd(p, a->dtype, a->D, mode, false, s), "t5a_fwd_sparse");
 }
 

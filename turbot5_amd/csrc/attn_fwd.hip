@@ -96,7 +96,11 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 template <typename T> struct Elem;
 template <> struct Elem<__bf16> {
-    using v8 = bf16x8; using v4 = bf16x4;
+    using v8 = bf16x8; using v4 = bf16x4; using v2 = bf16x2;
+    static __device__ __forceinline__ float sum2(v2 x, float acc) {
+        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(x, one, acc, false);
+    }
     static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
@@ -117,7 +121,11 @@ template <> struct Elem<__bf16> {
     }
 };
 template <> struct Elem<_Float16> {
-    using v8 = f16x8; using v4 = f16x4;
+    using v8 = f16x8; using v4 = f16x4; using v2 = f16x2;
+    static __device__ __forceinline__ float sum2(v2 x, float acc) {
+        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(x, one, acc, false);
+    }
     static __device__ __forceinline__ f32x16 mfma(v8 a, v8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
@@ -137,7 +145,7 @@ template <> struct Elem<_Float16> {
     }
 };
 template <> struct Elem<float> {
-    using v8 = float; using v4 = f32x4;   // operands of the fp32 MFMA are one float per lane
+    using v8 = float; using v4 = f32x4; using v2 = float;   // operands of the fp32 MFMA are one float per lane
     static __device__ __forceinline__ f32x16 mfma(float a, float b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
     }
@@ -339,7 +347,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // Fetch the launch parameters every path needs in one go: left alone, the compiler loads each
     // field just before its first use, which puts a chain of dependent scalar-load round trips on the
     // critical path of every workgroup.
-    asm volatile("" :: "s"(p.total_items), "s"(p.tiles_per_seq), "s"(p.H), "s"(p.M), "s"(p.N), "s"(p.nsplit),
+    asm volatile("" :: "s"(p.total_items), "s"(p.tiles_per_seq), "s"(p.H), "s"(p.M), "s"(p.N), "s"(p.nsplit), "s"(p.block_items),
                  "s"(p.align_end), "s"(p.c1), "s"(p.cu_q), "s"(p.plan), "s"(p.table), "s"(p.table_dtype));
     asm volatile("" :: "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.o), "s"(p.q_sb), "s"(p.q_sh), "s"(p.q_sr),
                  "s"(p.k_sb), "s"(p.k_sh), "s"(p.k_sr), "s"(p.v_sb), "s"(p.v_sh), "s"(p.v_sr));
@@ -364,7 +372,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         const unsigned wi = (ga + (k - level * gx)) * tps + level;
         if (wi < lo || wi >= hi) return;
         w = (int)wi;
-    } else if (BLOCK && p.nsplit > 1) {
+    } else if (BLOCK && p.block_items > 0) {
+        // (block_items > 0 marks the launch that carries the global rows' key splits, however many splits there are)
         // the key splits of the global rows are the longer items: they take the first workgroup ids, so that they
         // start first and the block items fill in around them; the block items follow in per-XCD slices
         const int n_split = p.total_items - p.block_items;
@@ -391,7 +400,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     if constexpr (RUNS) {
         run_next = w * p.run_len;
         run_left = min(p.run_len, p.tiles_per_seq * p.H * p.B - run_next);
-        if (BLOCK && p.nsplit > 1 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
+        if (BLOCK && p.block_items > 0 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
     }
     for (;;) {
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
@@ -440,7 +449,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         unsigned bh = (tps & (tps - 1)) == 0 ? entry >> __builtin_ctz(tps | 0x80000000u) : entry / tps;
         qt = (int)(entry - bh * tps);
         if (CAUSAL) qt = p.tiles_per_seq - 1 - qt;
-        if (BLOCK && p.nsplit > 1 && w >= p.block_items) {
+        if (BLOCK && p.block_items > 0 && w >= p.block_items) {
             // block pattern, behind the block items: key split `split` of the global rows of one (batch, head) --
             // its first G rows attend all keys, standard bias; the partial results are merged by a second kernel
             gsplit = true;
@@ -1651,6 +1660,131 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             head_refill = head_raise(st_next, mh, live & head_trigger(mh));
         }
     };
+    // Dense and packed modes at head_dim 64: the fast step without row maxima.
+    //
+    // The vector port, not the matrix pipe, bounds the step (per tile and wavefront: 32 exponentials at half rate,
+    // 16 conversions, 16 row-sum instructions and the issue slots of 16 matrix products), so the 19 instructions of
+    // the row maximum are worth removing, and the exponentials are worth spreading evenly over all sixteen products
+    // instead of sitting beside eight of them:
+    //  * No maximum.  The running max may lag behind by 2^24 anyway (raise_limit), and fp32 holds 2^127: whether it
+    //    must be raised follows from the tile's row SUM, which the step forms anyway -- a lane's sum of 32
+    //    probabilities above 2^24 (2^14 for fp16) means one of them is above 2^19, and only then the exact maximum is
+    //    looked up (rare block below), the running max raised and the tile's exponentials formed again from its
+    //    scores, which are still in registers.  The test comes BEFORE the tile's PV products, so an overflowing
+    //    exponential (inf) never reaches the output accumulators, whatever the inputs.  No probability above the
+    //    limit reaches the matrix core: without the trigger every one of them is at most the lane's sum.
+    //  * A tile's exponentials in two halves: those of its first 32 keys beside the PV products of the tile before
+    //    it (second half of the previous step, as soon as its scores exist), those of its last 32 keys beside the
+    //    S products of the tile after it (first half of its own step).  Every product then has two exponentials,
+    //    one conversion and one sum instruction beside it: 25 vector cycles against the product's 32.
+    // Rows: every row that will ever see a key has seen one in tile 0 (the prologue's head is the exact one), so the
+    // fast steps never start a row; a row without keys has scores of -inf, sums of 0 and never triggers.
+    // State between the steps: pe = the packed probabilities of the early half of the tile whose scores wait in
+    // registers, lt0 / lt1 = its partial row sums (kept apart from l_run until the tile has passed its test).
+    constexpr bool V2 = false && DENSE && DMA && D == 64;
+    unsigned pe[8];
+    float lt0 = 0.f, lt1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pe[j] = 0u;
+    // two exponentials, packed, and added to a partial sum
+    auto exp_pair = [&](float a, float b, float& acc) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        using v2 = typename E::v2;
+        if constexpr (!F32) {
+            const f32x2 e = {__builtin_amdgcn_exp2f(a), __builtin_amdgcn_exp2f(b)};
+            const v2 pk = __builtin_convertvector(e, v2);
+            acc = E::sum2(pk, acc);
+            return __builtin_bit_cast(unsigned, pk);
+        } else {
+            return 0u;
+        }
+    };
+    // entering a run of fast steps: the early half of the tile in `st` (its head has been done: no test needed)
+    auto dense_enter = [&](const f32x16 (&st)[NT]) {
+        if constexpr (V2) {
+            lt0 = 0.f; lt1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pe[j] = exp_pair(st[0][2 * j], st[0][2 * j + 1], (j & 1) ? lt1 : lt0);
+        }
+    };
+    auto dense_halves = [&](int vstage, const v8 (&ka)[NT][KS], f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        if constexpr (V2) {
+            static_assert(!V2 || (NT == 2 && KS == 4 && DT == 2), "four groups of 16 keys, two products each");
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const T* vs = Vs + vstage * V_TILE;
+            unsigned pl[8];     // packed probabilities of the late half of tile t
+            v8 vf[4][DT];       // V^T fragments
+            auto vread = [&](int g, int dt) {
+                const T* a0 = vs + vtr_off[dt] + 16 * g * D;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a0 + 8 * D));
+                vf[g][dt] = __builtin_bit_cast(v8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            };
+            __builtin_amdgcn_sched_barrier(0);
+            // first half: the late exponentials of tile t beside the S products of tile t+1
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pl[i] = exp_pair(st[1][2 * i], st[1][2 * i + 1], (i & 1) ? lt1 : lt0);
+                if (i >= 2) st_next[i & 1] = E::mfma(ka[i & 1][i >> 1], qf[i >> 1], st_next[i & 1]);
+                if (i >= 4) vread((i - 4) >> 1, (i - 4) & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (exact) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) st_next[nt][r] *= p.c1;
+            }
+            // tile t's test: a lane's sum above the limit
+            float lt = lt0 + lt1;
+            if (__any(lt > __builtin_amdgcn_exp2f(raise_limit<T>()))) {
+                asm volatile("");   // keep this rare block a real branch
+                const float mx = xhalf_max(head_max(st));
+                // (a triggering lane holds a probability above limit - 5: its row is raised)
+                const bool raise = mx > raise_limit<T>() - 6.0f;
+                const float delta = raise ? mx : 0.f;
+                const float scale = __builtin_amdgcn_exp2f(-delta);
+                m_run += delta;
+                m_zero = m_zero && !__any(raise);
+                l_run *= scale;
+                l_alt *= scale;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) { st[nt][r] -= delta; st_next[nt][r] -= delta; }
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) ot[dt][r] *= scale;
+                lt0 = 0.f; lt1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    pe[j] = exp_pair(st[0][2 * j], st[0][2 * j + 1], (j & 1) ? lt1 : lt0);
+                    pl[j] = exp_pair(st[1][2 * j], st[1][2 * j + 1], (j & 1) ? lt1 : lt0);
+                }
+                lt = lt0 + lt1;
+                head_refill = true;
+            }
+            l_run += lt;
+            lt0 = 0.f; lt1 = 0.f;
+            __builtin_amdgcn_sched_barrier(0);
+            // second half: PV products of tile t beside the early exponentials of tile t+1
+            unsigned pn[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int g = i >> 1, dt = i & 1;
+                const u32x4 pw = g < 2 ? u32x4{pe[4 * g], pe[4 * g + 1], pe[4 * g + 2], pe[4 * g + 3]}
+                                       : u32x4{pl[4 * g - 8], pl[4 * g - 7], pl[4 * g - 6], pl[4 * g - 5]};
+                ot[dt] = E::mfma(vf[g][dt], __builtin_bit_cast(v8, pw), ot[dt]);
+                if (i < 4) vread(2 + (i >> 1), i & 1);
+                pn[i] = exp_pair(st_next[0][2 * i], st_next[0][2 * i + 1], (i & 1) ? lt1 : lt0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pe[j] = pn[j];
+        }
+    };
     // Fast step (LDS-DMA path): tiles t and t+1 are neither skipped nor masked, so the step is the
     // general one minus those cases.  ST is the step index modulo 4, which fixes every LDS stage at
     // compile time.
@@ -1692,7 +1826,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 st_next[0] = E::mfma(ka[0][0], qf[0], cm);   // cm stays live: untied accumulator input
                 st_next[1] = E::mfma(ka[1][0], qf[0], cm);
             }
-            fused_halves(live, ST, ka, st, st_next);
+            if constexpr (V2) dense_halves(ST, ka, st, st_next);
+            else fused_halves(live, ST, ka, st, st_next);
         } else {
             __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): one wait for all K fragments instead of one per MFMA
             compute_s(nx, (ST + 1) & 3, ka, st_next);
@@ -1827,6 +1962,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     if constexpr (DENSE) { cursor_seek(t + 4, t + 3); fc_until = 0; }
                 }
                 if (quads > 0) T5A_PHASE_START();
+                const bool ran_fast = quads > 0;
+                if (V2 && ran_fast) dense_enter(sta);
                 while (quads > 0) {
                     fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
                     fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
@@ -1834,6 +1971,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
                     --quads; t += 4;
                 }
+                // (the dense fast steps leave the tile that follows them without its head: the general step wants
+                // it done; its early exponentials are simply formed again there)
+                if (V2 && ran_fast && !tc.skip) head_refill = softmax_head(tc, sta) || head_refill;
                 if (t >= ntiles) break;
             }
             step(t, sta, stb);
@@ -1941,7 +2081,7 @@ static hipError_t launch_exact(const FwdParams& p, hipStream_t stream) {
         }
     }
     unsigned grid = (unsigned)(((p.total_items + 7) / 8) * 8);
-    if ((MODE == kBlock || MODE == kBlockBits) && p.nsplit > 1)
+    if ((MODE == kBlock || MODE == kBlockBits) && p.block_items > 0)
         grid = (unsigned)(((p.total_items - p.block_items + 7) / 8) * 8 + ((p.block_items + 7) / 8) * 8);
     if (MODE == kPacked && p.plan != nullptr) grid = 8u * (unsigned)p.plan_slots;
     if (CAUSAL && MODE == kDense && p.xcd_lo[8] > 0) {

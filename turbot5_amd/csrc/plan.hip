@@ -261,12 +261,20 @@ bool plan_can_stage(int slots, int H, int max_seqlen_q) {
 
 hipError_t launch_varlen_plan(const PlanParams& p, hipStream_t stream) {
     const size_t dyn = p.staged ? (size_t)8 * p.slots * sizeof(int) : 0;
-    static std::atomic<size_t> granted{0};
-    if (dyn > granted.load(std::memory_order_relaxed)) {   // static + dynamic LDS beyond 64 KB must be allowed first
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(varlen_plan_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+    // per device: largest dynamic LDS size already allowed (the attribute belongs to the function as loaded on one device)
+    constexpr int kMaxDevices = 64;
+    static std::atomic<size_t> granted[kMaxDevices] = {};
+    if (dyn > 0) {   // static + dynamic LDS beyond 64 KB must be allowed first
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
-        granted.store(dyn, std::memory_order_relaxed);
+        const bool known = dev >= 0 && dev < kMaxDevices;
+        if (!known || dyn > granted[dev].load(std::memory_order_relaxed)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(varlen_plan_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+            if (e != hipSuccess) return e;
+            if (known) granted[dev].store(dyn, std::memory_order_relaxed);
+        }
     }
     hipLaunchKernelGGL(varlen_plan_kernel, dim3(1), dim3(PLAN_THREADS), dyn, stream, p);
     return hipGetLastError();

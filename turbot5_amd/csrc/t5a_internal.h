@@ -31,6 +31,7 @@ enum Mode { kDense = 0, kLocal = 1, kBlock = 2, kTGlobal = 3, kPacked = 4, kLoca
 // widest sliding window that is folded into the distance LUT (the LUT then spans 2 * (window + 96) distances;
 // 256 keeps it below 12 KB of LDS, so that two workgroups still share a compute unit)
 constexpr int kMaxLutWindow = 256;
+constexpr int kMaxRunLen = 16;     // most q tiles of one (batch, head) that a sparse work item takes
 constexpr int kKeyBitsFront = 8;   // zero words in front of a sequence's validity bits (tiles start up to 255 keys early)
 
 struct FwdParams {

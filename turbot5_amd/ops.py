@@ -24,12 +24,37 @@ _DTYPES = {torch.bfloat16: L.T5A_BF16, torch.float32: L.T5A_F32, torch.float16: 
 # False: the query rows are multiplied by sm_scale * log2(e) and rounded back to the input type before the
 # matrix product (relative error 2^-9 per term in bf16; still 3.6 times more accurate than the reference's
 # 'basic' path in bf16, and within 2e-2 of fp32 math for scores of deviation up to about 4).  True: the factor
-# is applied to the fp32 product, as the reference's fused kernel does; about 11 % slower at head_dim 64.
+# is applied to the fp32 product, as the reference's fused kernel does (one more multiply per score).
+# "prescaled" (per call only): q already carries sm_scale * log2(e), see ``prescaled_query``; the kernel applies
+# no factor, so q was rounded to its type once -- the accuracy of True at the speed of False.
 EXACT_SCORES = False
+LOG2E = 1.4426950408889634
+
+# Sparse patterns: q tiles per work item (0: the library chooses from the shape and the device).  Results do not
+# depend on it; tests pin every path of the run logic with it.
+RUN_LEN = 0
 
 
 def _exact(flag) -> int:
+    if isinstance(flag, str):
+        if flag != "prescaled":
+            raise ValueError(f"exact_scores={flag!r}: None, False, True or 'prescaled'")
+        return L.SCORES_PRESCALED
     return int(EXACT_SCORES if flag is None else bool(flag))
+
+
+def prescaled_query(hidden: torch.Tensor, weight: torch.Tensor, dtype: torch.dtype, sm_scale: float = 1.0) -> torch.Tensor:
+    """The query projection with sm_scale * log2(e) folded in: ``hidden @ weight.T * (sm_scale * log2 e)`` rounded to
+    ``dtype`` ONCE, for ``exact_scores="prescaled"``.  Activations that are already in ``dtype`` take the factor
+    as the GEMM's alpha (applied to the fp32 accumulator, before the rounding of the output); wider activations
+    are multiplied on their way into the cast."""
+    c = float(sm_scale) * LOG2E
+    x2 = hidden.reshape(-1, hidden.shape[-1])
+    if x2.dtype == dtype and weight.dtype == dtype:
+        q = torch.addmm(x2.new_zeros(1), x2, weight.t(), beta=0, alpha=c)
+    else:
+        q = torch.mul(torch.nn.functional.linear(x2, weight), c).to(dtype)
+    return q.view(*hidden.shape[:-1], weight.shape[0])
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -393,6 +418,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
     a.pattern, a.block_len, a.aux = pattern, int(block_len), int(aux)
     a.sm_scale = float(sm_scale)
     a.exact_scores = _exact(exact_scores)
+    a.run_len = int(RUN_LEN)
     if seq_lens is not None:
         a.seq_lens = seq_lens.data_ptr()
     if seq_starts is not None:
