@@ -1681,7 +1681,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // fast steps never start a row; a row without keys has scores of -inf, sums of 0 and never triggers.
     // State between the steps: pe = the packed probabilities of the early half of the tile whose scores wait in
     // registers, lt0 / lt1 = its partial row sums (kept apart from l_run until the tile has passed its test).
-    constexpr bool V2 = false && DENSE && DMA && D == 64;
+    constexpr bool V2 = DENSE && DMA && D == 64;
     unsigned pe[8];
     float lt0 = 0.f, lt1 = 0.f;
 #pragma unroll
@@ -1781,8 +1781,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 pn[i] = exp_pair(st_next[0][2 * i], st_next[0][2 * i + 1], (i & 1) ? lt1 : lt0);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // (pinned here: the compiler otherwise sinks the last step's exponentials of an unrolled group of four
+            // to the loop's back edge, away from the products they are meant to run beside)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) pe[j] = pn[j];
+            for (int j = 0; j < 8; ++j) { pe[j] = pn[j]; asm volatile("" : "+v"(pe[j])); }
+            asm volatile("" : "+v"(lt0), "+v"(lt1));
         }
     };
     // Fast step (LDS-DMA path): tiles t and t+1 are neither skipped nor masked, so the step is the
