@@ -23,7 +23,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                         difference between what the timed launches wrote and that CPU path on row subsets
 
 --leg NAME runs one kernel K times and nothing else, for profiling:
-    dense:BxL[c]  local  block  tglobal  splitk  varlen  varlen_causal  copy
+    dense:BxL[c][:exact|:prescaled]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
 --leg NAME --timeline does the same with the measurement build of the library (`python -m turbot5_amd.build --trace`)
 and prints where the work items of the last launch spent their shader-clock cycles.
 """
@@ -39,6 +39,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_F32_TFLOPS = 157.3     # MI355X dense fp32 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "fwd_kernel_bf16_d64_dense_B16_L1024.hbm_traffic.txt")
 B, H, L, D = 16, 12, 1024, 64
@@ -202,6 +203,25 @@ def extra_workloads(torch, dev, steps, samples):
                                                  "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
         samples.append(dense_sample(torch, f"dense_causal_B{bsz}_L{ln}", q, k, v, table, f(), True, bsz - 1, 3, 32))
         del q, k, v
+
+    # ---- score precision modes at the headline shape and at L = 16384: the default (Q * log2 e rounded to bf16 in
+    # the kernel), exact (the factor applied to the fp32 product) and prescaled (what the attention modules do: the
+    # factor folded into the query projection, nothing applied in the kernel)
+    modes = {}
+    for bsz, ln in ((B, L), (1, 16384)):
+        q, k, v, table = make_inputs(torch, dev, bsz, H, ln, D, seed=ln if ln != L else 0)
+        qs = (q.float() * ops.LOG2E).to(q.dtype)
+        for mode, qq, arg in (("default", q, None), ("exact", q, True), ("prescaled", qs, "prescaled")):
+            f = lambda: ops.flash_attention_with_fusing_bias(qq, k, v, table, causal=False, sm_scale=1.0, exact_scores=arg)  # noqa: E731
+            _, ms = time_kernel(torch, f, reps, warm)
+            tf = 4.0 * bsz * H * D * ln * ln / (ms * 1e-3) / 1e12
+            modes[f"B{bsz}_L{ln}_{mode}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+            if mode != "default":
+                # (prescaled: the oracle gets the rows the kernel was given, divided by log2 e again)
+                qref = qq if mode == "exact" else (qq.float() / ops.LOG2E)
+                samples.append(dense_sample(torch, f"dense_B{bsz}_L{ln}_{mode}", qref, k, v, table, f(), False, bsz - 1, 2, 34))
+        del q, k, v, qs
+    out["score_modes"] = modes
 
     # ---- head_dim 128 (the T5-3B / 11B head shape): B4 H6 L4096, same FLOPs as the B4 H12 D64 sweep point
     g = torch.Generator().manual_seed(6)
@@ -405,8 +425,9 @@ def check_sample(torch, O, s):
 
 def cpu_baseline(torch, samples, seconds_budget=24.0):
     """The oracle's 'basic' path (materialised bias, einsum, fp32 softmax, einsum) on the host cores: bounded
-    samples of the headline workload (C2), of the packed batch (C3) and the T5-small encoder (C1); and the
-    checks of the timed GPU launches.  This function is the only place where bench.py uses the oracle."""
+    samples of the headline workload (C2), of the packed batch (C3), the T5-small encoder (C1), the sparse patterns
+    at L = 16384 (C4, one head) and the decode shape (C5, 8 of 64 batch elements); and the checks of the timed GPU
+    launches.  This function is the only place where bench.py uses the oracle."""
     from oracle import t5_basic as O
     from oracle import t5_model as OM
     torch.set_num_threads(os.cpu_count() or 1)
@@ -449,6 +470,32 @@ def cpu_baseline(torch, samples, seconds_budget=24.0):
     OM.encoder_forward(sd, cfg, ids)
     dt = time.perf_counter() - t0
     other["t5_small_encoder_B4_L512_fp32"] = {"ms": round(dt * 1e3, 1), "tokens_per_s": round(2048 / dt, 1)}
+    # C4: the three sparse patterns at the full L = 16384, one head each (the oracle's blocked evaluation
+    # materialises the bias and mask per block, as the reference's modules do)
+    Ls = SPARSE_L
+    qs, ks, vs = (0.5 * torch.randn(1, 1, Ls, D, generator=g) for _ in range(3))
+    t1 = table[:, :1]
+    sk, sv = (0.5 * torch.randn(1, 1, Ls // 16, D, generator=g) for _ in range(2))
+    for name, fn, pairs in (
+            ("local_r127", lambda: O.local_attention_blocked(qs, ks, vs, t1, 128), Ls * 255 - 127 * 128),
+            ("block_128_g64", lambda: O.block_attention_blocked(qs, ks, vs, t1, 128, 64), 64 * Ls + (Ls - 64) * 192 - 64 * 64),
+            ("tglobal_r127_g16", lambda: O.tglobal_attention_blocked(qs, ks, vs, sk, sv, t1, 128, 16),
+             Ls * 255 - 127 * 128 + Ls * (Ls // 16))):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        other[f"sparse_{name}_one_head_L{Ls}"] = {"ms": round(dt * 1e3, 1), "heads_timed": 1, "of_heads": H,
+                                                 "tflops_live_pairs": round(4.0 * D * pairs / dt / 1e12, 4)}
+    # C5 decode: one query row over an 8192-token memory, 8 of the 64 batch elements, 12 heads, no bias
+    qd = 0.5 * torch.randn(8, H, 1, D, generator=g)
+    kd, vd = (0.5 * torch.randn(8, H, 8192, D, generator=g) for _ in range(2))
+    O.basic_attention(qd, kd, vd, None)
+    t0 = time.perf_counter()
+    O.basic_attention(qd, kd, vd, None)
+    dt = time.perf_counter() - t0
+    other["cross_attention_layer_step_B8_of_64_N8192"] = {
+        "ms": round(dt * 1e3, 2), "gbytes_per_s_bf16_equivalent": round(2 * 8 * 8192 * 768 * 2 / dt / 1e9, 2),
+        "note": "fp32 'basic' on the host; bytes counted as the bf16 cache the GPU kernel reads"}
     res["other_workloads"] = other
     res["checks"] = {s.name: round(check_sample(torch, O, s), 5) for s in samples}
     res["checks_note"] = ("max-abs of (what the timed launch wrote) - ('basic' math in fp32 on the same bf16 inputs) over "
@@ -467,13 +514,24 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
             y.copy_(x)
         torch.cuda.synchronize()
         return {"leg": "copy", "bytes_per_copy": x.numel()}
+    peak = PEAK_BF16_TFLOPS
     if name.startswith("dense:"):
-        shape = name.split(":", 1)[1]
+        parts = name.split(":")
+        shape, mode = parts[1], (parts[2] if len(parts) > 2 else None)
         causal = shape.endswith("c")
         b, l = (int(x) for x in shape.rstrip("c").split("x"))
         q, k, v, table = make_inputs(torch, dev, b, H, l, D, seed=l if (b, l) != (B, L) else 0)
-        f = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0)  # noqa: E731
+        exact = {None: None, "exact": True, "prescaled": "prescaled"}[mode]
+        f = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0, exact_scores=exact)  # noqa: E731
         fl = 4.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
+    elif name == "dense_f32_c1":
+        # the attention of baseline configuration 1 (T5-small encoder): B4 H8 L512 D64 in fp32, on the fp32 matrix cores
+        g = torch.Generator().manual_seed(3)
+        q, k, v = ((0.5 * torch.randn(4, 8, 512, 64, generator=g)).to(dev) for _ in range(3))
+        table = torch.randn(32, 8, generator=g).to(dev)
+        f = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0)  # noqa: E731
+        fl = 4.0 * 4 * 8 * 512 * 512 * 64
+        peak = PEAK_F32_TFLOPS
     elif name in ("local", "block", "tglobal"):
         q, k, v, table, sk, sv = sparse_inputs(torch, dev)
         if name == "local":
@@ -504,7 +562,7 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
                "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
     else:
         out = {"leg": name, "kernel_ms": round(ms, 5), "tflops": round(fl / ms / 1e9, 1),
-               "frac_mfma_peak": round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+               "frac_mfma_peak": round(fl / ms / 1e9 / peak, 4), "mfma_peak_tflops": peak}
     if timeline:
         out["timeline"] = read_timeline(torch, f)
     return out
@@ -559,7 +617,7 @@ def main():
     ap.add_argument("--no-models", action="store_true", help="skip the T5-base model legs (encoder, 100k pass, decoding)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and its checks")
     ap.add_argument("--leg", default=None, metavar="NAME",
-                    help="run only one kernel: dense:BxL[c], local, block, tglobal, splitk, varlen, varlen_causal, copy")
+                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
     ap.add_argument("--timeline", action="store_true",
                     help="with --leg: use the measurement build (libt5attn_trace.so) and print the work items' cycle stamps")
     ap.add_argument("--full", action="store_true", help="accepted for compatibility: the default run is the full one")
