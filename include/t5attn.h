@@ -106,7 +106,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 113
+#define T5A_ABI_VERSION 114
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -139,6 +139,31 @@ typedef struct t5a_dense_args {
     t5a_bias bias;
 } t5a_dense_args;
 int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
+
+/*
+ * Backward of t5a_fwd_dense: dq, dk, dv and the gradient of the (num_buckets, H) bias table.
+ * Replaces flash_attn_v2_bwd_bias behind FlashAttentionBias.backward
+ * (src/turbot5/ops/fused_bias_attention.py:851-873; kernels :397-820, the table gradient's atomics :617-619).
+ * q, k, v, causal, sm_scale, exact_scores and bias as in the forward call; o and lse are what it returned
+ * (lse is required); dout is the gradient of o.  dq (B,H,M,D), dk and dv (B,H,N,D) in the tensors' type, any
+ * strides {batch, head, row}; dtable (required when bias.table is set): (num_buckets, H) contiguous fp32, overwritten.
+ * head_dim 16, 32 or 64.  All arithmetic is fp32 (fp32 matrix cores) whatever the tensors' type.  The table
+ * gradient is summed with floating-point atomics: its last bits depend on the order of the workgroups.
+ * workspace: t5a_bwd_workspace_bytes(B, H, M) bytes of 16-byte aligned device memory.
+ */
+typedef struct t5a_dense_bwd_args {
+    const void* q; const void* k; const void* v; const void* o; const void* dout; const float* lse;
+    void* dq; void* dk; void* dv; float* dtable;
+    void* workspace; int64_t workspace_bytes;
+    int64_t q_strides[3]; int64_t k_strides[3]; int64_t v_strides[3]; int64_t o_strides[3]; int64_t dout_strides[3];
+    int64_t dq_strides[3]; int64_t dk_strides[3]; int64_t dv_strides[3];
+    int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
+    int32_t causal; float sm_scale;
+    int32_t exact_scores; int32_t reserved;
+    t5a_bias bias;
+} t5a_dense_bwd_args;
+int64_t t5a_bwd_workspace_bytes(int32_t B, int32_t H, int32_t M);
+int t5a_bwd_dense(const t5a_dense_bwd_args* args, t5a_stream_t stream);
 
 /*
  * Packed variable-length forward.

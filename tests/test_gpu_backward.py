@@ -1,0 +1,170 @@
+"""Backward of the dense fused-bias forward (t5a_bwd_dense behind ops.FlashAttentionBias) against torch.autograd
+through the oracle's dense attention on the same seeded inputs: dq, dk, dv and the gradient of the
+(num_buckets, H) table.  fp32: 1e-4 relative to the gradient's scale; bf16 / fp16: 2e-2 relative to it (the
+oracle differentiates fp32 math on the rounded inputs; the kernels do the same and round only their results).
+Reference: src/turbot5/ops/fused_bias_attention.py:397-873."""
+import ctypes as C
+
+import pytest
+import torch
+
+from oracle import t5_basic as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def rnd(*shape, seed=0, scale=0.5, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(*shape, generator=g)).to(dtype)
+
+
+def oracle_grads(q, k, v, table, dout, causal, sm_scale):
+    """Causal attention with more queries than keys: the first M - N rows see no key.  Their output is zero and they
+    have no gradient; autograd through a softmax over -inf alone gives NaN instead, so the oracle is differentiated
+    on the rows that see keys (same positions: the queries end where the keys end) and the others get zeros."""
+    M, N = q.shape[2], k.shape[2]
+    skip = max(M - N, 0) if causal else 0
+    q, k, v = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    tb = table.float().clone().requires_grad_(True) if table is not None else None
+    out = O.dense_attention(q[:, :, skip:], k, v, tb, causal, sm_scale)
+    out.backward(dout.float()[:, :, skip:])
+    out = torch.cat([torch.zeros_like(q[:, :, :skip]), out.detach()], dim=2)
+    return out, q.grad, k.grad, v.grad, (tb.grad if tb is not None else None)
+
+
+def check(name, got, want, tol):
+    scale = max(want.abs().max().item(), 1e-6)
+    err = (got.float().cpu() - want).abs().max().item()
+    assert err <= tol * scale, f"{name}: max-abs {err} against a gradient scale of {scale}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,H,M,N,D", [(2, 3, 256, 256, 64), (1, 2, 200, 333, 64), (2, 2, 130, 70, 64),
+                                         (1, 2, 96, 160, 32), (1, 1, 64, 64, 16), (1, 2, 1, 300, 64)])
+def test_gradients_match_autograd_through_the_oracle(gpu_device, dtype, causal, B, H, M, N, D):
+    from turbot5_amd import ops
+    q, k, v = rnd(B, H, M, D, seed=1, dtype=dtype), rnd(B, H, N, D, seed=2, dtype=dtype), rnd(B, H, N, D, seed=3, dtype=dtype)
+    table = rnd(32, H, seed=4, scale=1.0)
+    dout = rnd(B, H, M, D, seed=5, scale=1.0, dtype=dtype)
+    want_o, wq, wk, wv, wt = oracle_grads(q, k, v, table, dout, causal, 1.0)
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    out = ops.flash_attention_with_fusing_bias(dq, dk, dv, dt, causal=causal, sm_scale=1.0)
+    assert (out.float().cpu() - want_o).abs().max().item() <= (1e-4 if dtype == torch.float32 else 2e-2)
+    out.backward(dout.to(gpu_device))
+    tol = TOL[dtype]
+    check("dq", dq.grad, wq, tol)
+    check("dk", dk.grad, wk, tol)
+    check("dv", dv.grad, wv, tol)
+    check("dtable", dt.grad, wt, tol)
+    assert dq.grad.dtype == dtype and dt.grad.dtype == torch.float32 and dq.grad.shape == q.shape
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_gradients_of_strided_views_without_a_table_and_with_a_scale(gpu_device, causal):
+    """(B, L, H, D) projections viewed as (B, H, L, D), as the modules hand them over; no bias table; 1/sqrt(d)."""
+    from turbot5_amd import ops
+    B, H, L, D = 2, 4, 192, 64
+    q, k, v = (rnd(B, L, H, D, seed=10 + i).transpose(1, 2) for i in range(3))
+    dout = rnd(B, L, H, D, seed=13, scale=1.0).transpose(1, 2)
+    want_o, wq, wk, wv, _ = oracle_grads(q, k, v, None, dout, causal, None)
+    dq, dk, dv = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    out = ops.flash_attention_with_fusing_bias(dq, dk, dv, None, causal=causal)
+    out.backward(dout.to(gpu_device))
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv)):
+        check(name, g, w, 1e-4)
+
+
+def test_gradients_with_prescaled_query_rows(gpu_device):
+    """exact_scores="prescaled": the rows carry log2(e), the score factor of the op is ln 2 -- and so is the
+    factor on dq and dk.  Differentiated through ops.prescaled_query down to the hidden states and the weight."""
+    from turbot5_amd import ops
+    B, H, L, D = 1, 2, 160, 64
+    x = rnd(B, L, H * D, seed=20)
+    w = rnd(H * D, H * D, seed=21, scale=(H * D) ** -0.5)
+    k, v = rnd(B, H, L, D, seed=22), rnd(B, H, L, D, seed=23)
+    table = rnd(32, H, seed=24, scale=1.0)
+    dout = rnd(B, H, L, D, seed=25, scale=1.0)
+    xo, wo = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    qo = (xo @ wo.T).view(B, L, H, D).transpose(1, 2)
+    O.dense_attention(qo, k, v, table, False, 1.0).backward(dout)
+    xd, wd = x.to(gpu_device).requires_grad_(True), w.to(gpu_device).requires_grad_(True)
+    qd = ops.prescaled_query(xd, wd, torch.float32).view(B, L, H, D).transpose(1, 2)
+    out = ops.flash_attention_with_fusing_bias(qd, k.to(gpu_device), v.to(gpu_device), table.to(gpu_device),
+                                               sm_scale=1.0, exact_scores="prescaled")
+    out.backward(dout.to(gpu_device))
+    check("dx", xd.grad, xo.grad, 2e-4)
+    check("dw", wd.grad, wo.grad, 2e-4)
+
+
+def test_rows_without_keys_and_the_raw_entry_point(gpu_device):
+    """Causal with more queries than keys: the first M - N rows see nothing, their gradient is zero and nothing is
+    NaN.  Called through the C ABI with guard rows around dq, dk, dv; bad arguments are refused."""
+    from turbot5_amd import _lib, ops
+    B, H, M, N, D = 1, 2, 200, 120, 64
+    q, k, v = rnd(B, H, M, D, seed=30), rnd(B, H, N, D, seed=31), rnd(B, H, N, D, seed=32)
+    table, dout = rnd(32, H, seed=33, scale=1.0), rnd(B, H, M, D, seed=34, scale=1.0)
+    _, wq, wk, wv, wt = oracle_grads(q, k, v, table, dout, True, 1.0)
+    dev = [t.to(gpu_device) for t in (q, k, v, table, dout)]
+    o, lse = ops.flash_attention_with_fusing_bias(*dev[:4], causal=True, sm_scale=1.0, return_lse=True)
+    assert torch.isinf(lse[0, 0, :M - N]).all()
+    guard = 7.0
+    bufs = {n: torch.full((B, H, r + 2, D), guard, device=gpu_device) for n, r in (("dq", M), ("dk", N), ("dv", N))}
+    dtab = torch.full((32, H), guard, device=gpu_device)
+    lib = _lib.load()
+    ws = torch.empty(int(lib.t5a_bwd_workspace_bytes(B, H, M)), dtype=torch.uint8, device=gpu_device)
+    a = _lib.T5ADenseBwdArgs()
+    a.q, a.k, a.v, a.o, a.dout, a.lse = (t.data_ptr() for t in (dev[0], dev[1], dev[2], o, dev[4], lse))
+    a.dq, a.dk, a.dv = (bufs[n][:, :, 1:-1].data_ptr() for n in ("dq", "dk", "dv"))
+    a.dtable = dtab.data_ptr()
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    for name, t in (("q_strides", dev[0]), ("k_strides", dev[1]), ("v_strides", dev[2]), ("o_strides", o),
+                    ("dout_strides", dev[4]), ("dq_strides", bufs["dq"]), ("dk_strides", bufs["dk"]), ("dv_strides", bufs["dv"])):
+        setattr(a, name, (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2)))
+    a.dtype, a.B, a.H, a.M, a.N, a.D = _lib.T5A_F32, B, H, M, N, D
+    a.causal, a.sm_scale = 1, 1.0
+    a.bias.table, a.bias.table_dtype = dev[3].data_ptr(), _lib.T5A_F32
+    a.bias.num_buckets, a.bias.max_distance = 32, 128
+    a.bias.stride_bucket, a.bias.stride_head = dev[3].stride(0), dev[3].stride(1)
+    stream = torch.cuda.current_stream(gpu_device).cuda_stream
+    _lib.check(lib.t5a_bwd_dense(C.byref(a), stream))
+    torch.cuda.synchronize()
+    for n, w in (("dq", wq), ("dk", wk), ("dv", wv)):
+        buf = bufs[n].cpu()
+        assert (buf[:, :, 0] == guard).all() and (buf[:, :, -1] == guard).all(), n
+        assert torch.isfinite(buf).all()
+        check(n, buf[:, :, 1:-1], w, 1e-4)
+    assert (bufs["dq"][:, :, 1:1 + M - N] == 0).all()
+    check("dtable", dtab, wt, 1e-4)
+    a.workspace_bytes = 8
+    assert lib.t5a_bwd_dense(C.byref(a), stream) < 0 and b"workspace" in lib.t5a_last_error()
+    a.workspace_bytes = ws.numel()
+    a.D = 128
+    assert lib.t5a_bwd_dense(C.byref(a), stream) < 0
+    a.D = D
+    a.dtable = None
+    assert lib.t5a_bwd_dense(C.byref(a), stream) < 0
+
+
+def test_module_trains_through_the_fused_attention(gpu_device):
+    """A T5FlashAttention module in training mode: gradients reach its projections and its bias table, and agree
+    with the same module differentiated through the oracle's attention."""
+    from turbot5_amd import T5ATTENTION_TYPES, T5Config
+    cfg = T5Config(vocab_size=32, d_model=128, d_kv=64, d_ff=256, num_layers=1, num_heads=2, dropout_rate=0.0)
+    torch.manual_seed(3)
+    mod = T5ATTENTION_TYPES["flash"](cfg, has_relative_attention_bias=True)
+    x = torch.randn(2, 150, 128)
+    sd = {n: p.detach().clone().requires_grad_(True) for n, p in mod.named_parameters()}
+
+    def heads(t):
+        return t.view(2, 150, 2, 64).transpose(1, 2)
+    q, k, v = (heads(x @ sd[f"{n}.weight"].T) for n in ("q", "k", "v"))
+    o = O.dense_attention(q, k, v, sd["relative_attention_bias.weight"], False, 1.0)
+    (o.transpose(1, 2).reshape(2, 150, 128) @ sd["o.weight"].T).square().sum().backward()
+    mod = mod.to(gpu_device).train()
+    out = mod(x.to(gpu_device))[0]
+    out.square().sum().backward()
+    for n, p in mod.named_parameters():
+        check(n, p.grad, sd[n].grad, 2e-4)

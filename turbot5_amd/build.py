@@ -25,6 +25,7 @@ UNITS = [
     ("rmsnorm.o", "rmsnorm.hip", []),
     ("plan.o", "plan.hip", []),
     ("lut.o", "lut.hip", []),
+    ("attn_bwd.o", "attn_bwd.hip", []),
     ("attn_fwd_bf16.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=0"]),
     ("attn_fwd_f32.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=1"]),
     ("attn_fwd_f16.o", "attn_fwd.hip", ["-DT5A_UNIT_DTYPE=2"]),

@@ -289,6 +289,77 @@ int t5a_fwd_dense(const t5a_dense_args* a, t5a_stream_t stream) {
     return finish(launch_fwd(p, a->dtype, a->D, kDense, a->causal != 0, (hipStream_t)stream), "t5a_fwd_dense");
 }
 
+int64_t t5a_bwd_workspace_bytes(int32_t B, int32_t H, int32_t M) {
+    if (B < 0 || H < 0 || M < 0) return -1;
+    return 2 * (int64_t)B * H * M * (int64_t)sizeof(float);
+}
+
+int t5a_bwd_dense(const t5a_dense_bwd_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    if (a->D == 128) return fail(T5A_ERR_HEAD_DIM, "the backward kernels hold a row's head_dim in registers: head_dim 16, 32 or 64");
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if (a->B < 0 || a->H <= 0 || a->M < 0 || a->N < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d M=%d N=%d", a->B, a->H, a->M, a->N);
+    if (a->B == 0) return T5A_OK;
+    struct { const char* name; const void* ptr; const int64_t* st; int rows; } ts[] = {
+        {"q", a->q, a->q_strides, a->M}, {"o", a->o, a->o_strides, a->M}, {"dout", a->dout, a->dout_strides, a->M},
+        {"dq", a->dq, a->dq_strides, a->M}, {"k", a->k, a->k_strides, a->N}, {"v", a->v, a->v_strides, a->N},
+        {"dk", a->dk, a->dk_strides, a->N}, {"dv", a->dv, a->dv_strides, a->N}};
+    for (auto& t : ts) {
+        if (t.rows == 0) continue;
+        if ((rc = check_tensor(t.name, t.ptr, t.st, 3, unit))) return rc;
+    }
+    if (a->M > 0 && a->lse == nullptr) return fail(T5A_ERR_NULL, "lse is NULL");
+    const int64_t need = t5a_bwd_workspace_bytes(a->B, a->H, a->M);
+    if (a->M > 0 && (a->workspace == nullptr || a->workspace_bytes < need))
+        return fail(T5A_ERR_WORKSPACE, "t5a_bwd_dense: workspace of %lld bytes needed, %lld given", (long long)need, (long long)a->workspace_bytes);
+    if (a->M > 0 && !aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+    if ((int64_t)a->B > 65535 || (int64_t)a->H > 65535) return fail(T5A_ERR_SHAPE, "B or H too large for the launch grid");
+    BwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.dout = a->dout; p.lse = a->lse;
+    p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
+    p.q_sb = a->q_strides[0]; p.q_sh = a->q_strides[1]; p.q_sr = a->q_strides[2];
+    p.k_sb = a->k_strides[0]; p.k_sh = a->k_strides[1]; p.k_sr = a->k_strides[2];
+    p.v_sb = a->v_strides[0]; p.v_sh = a->v_strides[1]; p.v_sr = a->v_strides[2];
+    p.o_sb = a->o_strides[0]; p.o_sh = a->o_strides[1]; p.o_sr = a->o_strides[2];
+    p.do_sb = a->dout_strides[0]; p.do_sh = a->dout_strides[1]; p.do_sr = a->dout_strides[2];
+    p.dq_sb = a->dq_strides[0]; p.dq_sh = a->dq_strides[1]; p.dq_sr = a->dq_strides[2];
+    p.dk_sb = a->dk_strides[0]; p.dk_sh = a->dk_strides[1]; p.dk_sr = a->dk_strides[2];
+    p.dv_sb = a->dv_strides[0]; p.dv_sh = a->dv_strides[1]; p.dv_sr = a->dv_strides[2];
+    p.B = a->B; p.H = a->H; p.M = a->M; p.N = a->N;
+    FwdParams f;
+    memset(&f, 0, sizeof(f));
+    if ((rc = score_mode(a->exact_scores, a->sm_scale, &f))) return rc;
+    p.c1 = f.c1;
+    if ((rc = fill_bias(a->bias, a->causal == 0, &f))) return rc;
+    p.table = f.table; p.table_dtype = f.table_dtype; p.t_sbucket = f.t_sbucket; p.t_shead = f.t_shead; p.bs = f.bs;
+    p.n_buckets = a->bias.table != nullptr ? a->bias.num_buckets : 0;
+    if (a->bias.table != nullptr && a->dtable == nullptr) return fail(T5A_ERR_NULL, "dtable is NULL (the forward had a bias table)");
+    if (p.n_buckets > 4 * kMaxThresholds) return fail(T5A_ERR_BUCKETS, "num_buckets=%d too large for the backward", p.n_buckets);
+    p.dtable = a->bias.table != nullptr ? a->dtable : nullptr;
+    if (a->M == 0) {
+        // no query rows: dk and dv are zero, and so is the table gradient
+        hipError_t e = hipSuccess;
+        if (a->N > 0) {
+            const size_t es = a->dtype == T5A_F32 ? 4 : 2;
+            for (void* out : {a->dk, a->dv}) {
+                const int64_t* st = out == a->dk ? a->dk_strides : a->dv_strides;
+                if (st[2] != a->D || st[1] != (int64_t)a->N * a->D || st[0] != (int64_t)a->H * a->N * a->D)
+                    return fail(T5A_ERR_STRIDE, "M == 0: dk and dv must be contiguous");
+                if (e == hipSuccess) e = hipMemsetAsync(out, 0, (size_t)a->B * a->H * a->N * a->D * es, (hipStream_t)stream);
+            }
+        }
+        if (e == hipSuccess && p.dtable != nullptr)
+            e = hipMemsetAsync(p.dtable, 0, (size_t)p.n_buckets * a->H * sizeof(float), (hipStream_t)stream);
+        return finish(e, "t5a_bwd_dense (no query rows)");
+    }
+    p.delta = reinterpret_cast<float*>(a->workspace);
+    p.lse2 = p.delta + (int64_t)a->B * a->H * a->M;
+    return finish(launch_bwd_dense(p, a->dtype, a->D, a->causal != 0, (hipStream_t)stream), "t5a_bwd_dense");
+}
+
 // Entries per XCD of a packed batch's launch plan: twice the mean, so that slices of equal work but
 // unequal item counts fit (a slice that still outgrows it spills into the others' free slots).
 static int plan_slots(int64_t items_bound) { return (int)(2 * ((items_bound + 7) / 8)); }

@@ -1,0 +1,319 @@
+// Backward of the dense fused-bias attention forward for gfx950: dq, dk, dv and the gradient of the
+// (num_buckets, H) bias table.  Replaces flash_attn_v2_bwd_bias of the reference
+// (src/turbot5/ops/fused_bias_attention.py:397-820: _bwd_preprocess, _bwd_kv_bias_kernel with its atomics on the
+// table gradient :617-619, _bwd_q_kernel).
+//
+// Three kernels, all arithmetic in fp32 (inputs of any of the three types are widened on their way into LDS; the
+// products run on the fp32 matrix cores, v_mfma_f32_32x32x2_f32), so one code path serves fp32 and 16-bit tensors
+// and the result does not depend on how the forward rounded its probabilities:
+//
+//   bwd_rows_kernel   delta_i = sum_d o_id do_id and the log-sum-exp in base-2 units, per query row; also clears the
+//                     table gradient
+//   bwd_kernel<KV=0>  a workgroup owns 128 query rows (32 per wavefront) and walks the key tiles of 64:
+//                     S^T = K Q^T, dP^T = V dO^T (key rows from LDS as the A operand, so a lane owns one query and
+//                     its log-sum-exp and delta are lane scalars), P^T = exp2(c1 S^T + bias - lse),
+//                     dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T.  The table gradient is collected here: tiles whose
+//                     distances are all saturated add their dS to one of two lane sums, the tiles around the
+//                     diagonal add element by element into a per-bucket histogram in LDS; one global atomic per
+//                     bucket and workgroup at the end.
+//   bwd_kernel<KV=1>  a workgroup owns 128 keys and walks the query tiles of 64, the same products with the roles
+//                     swapped (query rows from LDS; log-sum-exp and delta of the 64 queries staged in LDS):
+//                     dV^T += dO^T P, dK^T += Q^T dS.
+//
+// Scores use the key position j and the query position i + N - M, as the forward does; rows whose log-sum-exp is
+// -inf (no visible key) have no gradient.  Rows and keys past the end of a tensor are read as zeros and masked.
+#include "lut_device.h"
+#include "t5a_internal.h"
+
+namespace t5a {
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBwdThreads = 256;
+constexpr int kBwdOwn = 128;     // own rows per workgroup (queries for dq, keys for dk / dv)
+constexpr int kBwdOther = 64;    // rows of the other kind per tile
+constexpr int kMaxBuckets = 2 * 2 * kMaxThresholds;
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return static_cast<float>(x); }
+
+// four consecutive elements of a row as floats (8 or 16 bytes, aligned: head_dim and strides are multiples of 8 / 4)
+template <typename T> __device__ __forceinline__ f32x4 load4(const T* p) {
+    if constexpr (sizeof(T) == 4) {
+        return *reinterpret_cast<const f32x4*>(p);
+    } else {
+        typedef T t4 __attribute__((ext_vector_type(4)));
+        const t4 x = *reinterpret_cast<const t4*>(p);
+        return f32x4{to_f32(x[0]), to_f32(x[1]), to_f32(x[2]), to_f32(x[3])};
+    }
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, f32x4 x) {
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4*>(p) = x;
+    } else {
+        typedef T t4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<t4*>(p) = t4{(T)x[0], (T)x[1], (T)x[2], (T)x[3]};
+    }
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_rows_kernel(const BwdParams p) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;     // (b, h, i) flattened
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    // the table gradient is accumulated with atomics by the dq kernel: clear it here, ahead of that launch
+    if (p.dtable != nullptr) {
+        const int64_t n = (int64_t)p.n_buckets * p.H;
+        for (int64_t x = row; x < n; x += (int64_t)gridDim.x * 256) p.dtable[x] = 0.f;
+    }
+    if (row >= rows) return;
+    const int i = (int)(row % p.M);
+    const int64_t bh = row / p.M;
+    const int h = (int)(bh % p.H), b = (int)(bh / p.H);
+    const T* o = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)i * p.o_sr;
+    const T* g = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + (int64_t)i * p.do_sr;
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < D / 4; ++c) {
+        const f32x4 x = load4(o + 4 * c), y = load4(g + 4 * c);
+        acc += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+    }
+    p.delta[row] = acc;
+    const float l = p.lse[row];
+    // a row without a visible key: +inf makes every exp2(score - lse2) of the row 0
+    p.lse2[row] = l == -INFINITY ? INFINITY : l * 1.4426950408889634f;
+}
+
+template <typename T, int D, bool CAUSAL, bool KV>
+__global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) {
+    constexpr int STR = D + 1;              // fp32 tile rows padded by one float
+    constexpr int DT = (D + 31) / 32;       // 32-row blocks of the transposed gradients
+    constexpr int KS = D / 2;               // k-steps of a product over head_dim
+    constexpr int NT = kBwdOther / 32;
+    __shared__ float ta[kBwdOther * STR + 32];     // K (dq) / Q (dk, dv) tile
+    __shared__ float tb[kBwdOther * STR + 32];     // V (dq) / dO (dk, dv) tile
+    __shared__ float rowstat[2 * kBwdOther];       // KV: lse2 and delta of the tile's queries
+    __shared__ float lut_bias[2 * kMaxSaturation + 1];   // bias * log2(e) per clamped distance
+    __shared__ int lut_bucket[KV ? 1 : 2 * kMaxSaturation + 1];
+    __shared__ float hist[KV ? 1 : kMaxBuckets];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, hh = lane >> 5;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int own_base = blockIdx.x * kBwdOwn;
+    const int own_row = own_base + wave * 32 + lr;
+    const int n_own = KV ? p.N : p.M, n_other = KV ? p.M : p.N;
+    const int P = p.N - p.M;                       // query i sits at key position i + P
+    const bool has_bias = p.table != nullptr;
+    const int sat = has_bias ? p.bs.sat : 0;
+
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+    const T* gp = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.do_sb + (int64_t)h * p.do_sh;
+    const int64_t stat_base = ((int64_t)b * p.H + h) * p.M;
+
+    // bias (and bucket) per clamped distance
+    if (has_bias) {
+        for (int x = tid; x <= 2 * sat; x += kBwdThreads) {
+            const int bk = bucket_of(p.bs, x - sat);
+            lut_bias[x] = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * 1.4426950408889634f;
+            if constexpr (!KV) lut_bucket[x] = bk;
+        }
+        if constexpr (!KV)
+            for (int x = tid; x < p.n_buckets; x += kBwdThreads) hist[x] = 0.f;
+    }
+
+    // own rows as B operands of the 32x32x2 products: lane (lr, hh) holds elements 2s + hh of its row
+    const bool own_ok = own_row < n_own;
+    float fa[KS], fb[KS];
+    {
+        const T* a = (KV ? kp + (int64_t)own_row * p.k_sr : qp + (int64_t)own_row * p.q_sr);
+        const T* c = (KV ? vp + (int64_t)own_row * p.v_sr : gp + (int64_t)own_row * p.do_sr);
+#pragma unroll
+        for (int s4 = 0; s4 < D / 4; ++s4) {
+            f32x4 x = {0.f, 0.f, 0.f, 0.f}, y = {0.f, 0.f, 0.f, 0.f};
+            if (own_ok) { x = load4(a + 4 * s4); y = load4(c + 4 * s4); }
+            fa[2 * s4] = hh ? x[1] : x[0]; fa[2 * s4 + 1] = hh ? x[3] : x[2];
+            fb[2 * s4] = hh ? y[1] : y[0]; fb[2 * s4 + 1] = hh ? y[3] : y[2];
+        }
+    }
+    float lse2_own = INFINITY, delta_own = 0.f;
+    if (!KV && own_ok) { lse2_own = p.lse2[stat_base + own_row]; delta_own = p.delta[stat_base + own_row]; }
+
+    // tiles of the other kind that can hold a visible pair
+    int t_lo = 0, t_hi = (n_other + kBwdOther - 1) / kBwdOther;
+    if (CAUSAL) {
+        if (!KV) t_hi = min(t_hi, max(0, (own_base + kBwdOwn - 1 + P) / kBwdOther + 1));   // keys j <= i + P
+        else t_lo = max(0, own_base - P) / kBwdOther;                                      // queries i >= j - P
+    }
+
+    f32x16 acc_a[DT], acc_b[DT];     // dQ^T or dK^T; dV^T
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc_a[dt][r] = 0.f; acc_b[dt][r] = 0.f; }
+    float sum_lo = 0.f, sum_hi = 0.f;   // dS of the tiles saturated on the left / on the right of the diagonal
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int o0 = t * kBwdOther;
+        __syncthreads();     // the previous tile's readers are done (and the LUT is written, first time round)
+        {
+            const T* a = KV ? qp : kp;
+            const T* c = KV ? gp : vp;
+            const int64_t a_sr = KV ? p.q_sr : p.k_sr, c_sr = KV ? p.do_sr : p.v_sr;
+            for (int idx = tid; idx < kBwdOther * (D / 4); idx += kBwdThreads) {
+                const int row = idx / (D / 4), c4 = idx % (D / 4);
+                f32x4 x = {0.f, 0.f, 0.f, 0.f}, y = {0.f, 0.f, 0.f, 0.f};
+                if (o0 + row < n_other) {
+                    x = load4(a + (int64_t)(o0 + row) * a_sr + 4 * c4);
+                    y = load4(c + (int64_t)(o0 + row) * c_sr + 4 * c4);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { ta[row * STR + 4 * c4 + e] = x[e]; tb[row * STR + 4 * c4 + e] = y[e]; }
+            }
+            if (KV && tid < 2 * kBwdOther) {
+                const int row = tid & (kBwdOther - 1);
+                float val = tid < kBwdOther ? INFINITY : 0.f;
+                if (o0 + row < n_other) val = tid < kBwdOther ? p.lse2[stat_base + o0 + row] : p.delta[stat_base + o0 + row];
+                rowstat[tid] = val;
+            }
+        }
+        __syncthreads();
+
+        f32x16 s[NT], dp[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { s[nt][r] = 0.f; dp[nt][r] = 0.f; }
+            const int row = 32 * nt + lr;
+#pragma unroll
+            for (int k2 = 0; k2 < KS; ++k2) {
+                s[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(ta[row * STR + 2 * k2 + hh], fa[k2], s[nt], 0, 0, 0);
+                dp[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tb[row * STR + 2 * k2 + hh], fb[k2], dp[nt], 0, 0, 0);
+            }
+        }
+
+        // wavefront-uniform: every pair of this wavefront's tile lies at a saturated distance on one side
+        int side = 0;
+        if constexpr (!KV) {
+            const int i_lo = own_base + wave * 32 + P, i_hi = i_lo + 31;    // query positions
+            if (o0 + kBwdOther - 1 - i_lo <= -sat) side = 1;
+            else if (o0 - i_hi >= sat) side = 2;
+        }
+        float tile_sum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ol = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);   // row of the other kind inside the tile
+                const int i = KV ? o0 + ol : own_row, j = KV ? own_row : o0 + ol;
+                const int rel = j - (i + P);
+                const bool valid = i < p.M && j < p.N && (!CAUSAL || rel <= 0);
+                const int x = min(max(rel, -sat), sat) + sat;
+                const float bias2 = has_bias ? lut_bias[x] : 0.f;
+                const float l2 = KV ? rowstat[ol] : lse2_own;
+                const float dl = KV ? rowstat[kBwdOther + ol] : delta_own;
+                const float pv = valid ? __builtin_amdgcn_exp2f(__builtin_fmaf(p.c1, s[nt][r], bias2) - l2) : 0.f;
+                const float ds = pv * (dp[nt][r] - dl);
+                s[nt][r] = pv;
+                dp[nt][r] = ds;
+                if constexpr (!KV) {
+                    if (has_bias) {
+                        if (side != 0) tile_sum += ds;
+                        else if (valid) atomicAdd(&hist[lut_bucket[x]], ds);
+                    }
+                }
+            }
+        if (side == 1) sum_lo += tile_sum; else if (side == 2) sum_hi += tile_sum;
+
+        // dQ^T += K^T dS^T   /   dK^T += Q^T dS, dV^T += dO^T P   (contraction over the tile's 64 rows, two per product)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ol = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    acc_a[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(ta[ol * STR + 32 * dt + lr], dp[nt][r], acc_a[dt], 0, 0, 0);
+                    if constexpr (KV)
+                        acc_b[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tb[ol * STR + 32 * dt + lr], s[nt][r], acc_b[dt], 0, 0, 0);
+                }
+            }
+    }
+
+    // rows: lane (lr, hh) holds, for its own row, elements 32 dt + 8 g + 4 hh .. + 3 of the transposed gradients
+    const float scale = p.c1 * 0.6931471805599453f;     // d score / d (q . k), natural units
+    if (own_ok) {
+        T* oa = KV ? reinterpret_cast<T*>(p.dk) + (int64_t)b * p.dk_sb + (int64_t)h * p.dk_sh + (int64_t)own_row * p.dk_sr
+                   : reinterpret_cast<T*>(p.dq) + (int64_t)b * p.dq_sb + (int64_t)h * p.dq_sh + (int64_t)own_row * p.dq_sr;
+        T* ob = KV ? reinterpret_cast<T*>(p.dv) + (int64_t)b * p.dv_sb + (int64_t)h * p.dv_sh + (int64_t)own_row * p.dv_sr : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d0 = 32 * dt + 8 * g + 4 * hh;
+                if (d0 < D) {
+                    store4(oa + d0, f32x4{acc_a[dt][4 * g] * scale, acc_a[dt][4 * g + 1] * scale,
+                                          acc_a[dt][4 * g + 2] * scale, acc_a[dt][4 * g + 3] * scale});
+                    if constexpr (KV)
+                        store4(ob + d0, f32x4{acc_b[dt][4 * g], acc_b[dt][4 * g + 1], acc_b[dt][4 * g + 2], acc_b[dt][4 * g + 3]});
+                }
+            }
+    }
+    if constexpr (!KV) {
+        if (has_bias && p.dtable != nullptr) {
+            // the saturated tiles' sums: one value per wavefront and side, into the last bucket of that side
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                sum_lo += __shfl_xor(sum_lo, off, 64);
+                sum_hi += __shfl_xor(sum_hi, off, 64);
+            }
+            if (lane == 0) {
+                if (sum_lo != 0.f) atomicAdd(&hist[lut_bucket[0]], sum_lo);
+                if (sum_hi != 0.f) atomicAdd(&hist[lut_bucket[2 * sat]], sum_hi);
+            }
+            __syncthreads();
+            for (int x = tid; x < p.n_buckets; x += kBwdThreads)
+                if (hist[x] != 0.f) atomicAdd(&p.dtable[(int64_t)x * p.H + h], hist[x]);
+        }
+    }
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_d(const BwdParams& p, bool causal, hipStream_t stream) {
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    hipLaunchKernelGGL((bwd_rows_kernel<T, D>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const dim3 gq((p.M + kBwdOwn - 1) / kBwdOwn, p.H, p.B), gk((p.N + kBwdOwn - 1) / kBwdOwn, p.H, p.B);
+    if (causal) {
+        hipLaunchKernelGGL((bwd_kernel<T, D, true, false>), gq, dim3(kBwdThreads), 0, stream, p);
+        if (p.N > 0) hipLaunchKernelGGL((bwd_kernel<T, D, true, true>), gk, dim3(kBwdThreads), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((bwd_kernel<T, D, false, false>), gq, dim3(kBwdThreads), 0, stream, p);
+        if (p.N > 0) hipLaunchKernelGGL((bwd_kernel<T, D, false, true>), gk, dim3(kBwdThreads), 0, stream, p);
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_bwd_t(const BwdParams& p, int D, bool causal, hipStream_t s) {
+    switch (D) {
+        case 16: return launch_bwd_d<T, 16>(p, causal, s);
+        case 32: return launch_bwd_d<T, 32>(p, causal, s);
+        case 64: return launch_bwd_d<T, 64>(p, causal, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t launch_bwd_dense(const BwdParams& p, int dtype, int D, bool causal, hipStream_t stream) {
+    if (dtype == T5A_BF16) return launch_bwd_t<__bf16>(p, D, causal, stream);
+    if (dtype == T5A_F16) return launch_bwd_t<_Float16>(p, D, causal, stream);
+    if (dtype == T5A_F32) return launch_bwd_t<float>(p, D, causal, stream);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace t5a

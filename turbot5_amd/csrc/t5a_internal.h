@@ -125,6 +125,23 @@ struct PlanParams {
 bool plan_can_stage(int slots, int H, int max_seqlen_q);
 hipError_t launch_varlen_plan(const PlanParams& p, hipStream_t stream);
 
+// Backward of the dense forward (attn_bwd.hip)
+struct BwdParams {
+    const void* q; const void* k; const void* v; const void* o; const void* dout;
+    const float* lse;                 // (B,H,M) natural log-sum-exp of the forward
+    void* dq; void* dk; void* dv;
+    float* dtable;                    // (n_buckets, H) fp32, or null
+    float* delta; float* lse2;        // workspace, (B,H,M) each
+    int64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr, v_sb, v_sh, v_sr, o_sb, o_sh, o_sr, do_sb, do_sh, do_sr;
+    int64_t dq_sb, dq_sh, dq_sr, dk_sb, dk_sh, dk_sr, dv_sb, dv_sh, dv_sr;
+    int B, H, M, N;
+    float c1;                         // base-2 score factor: sm_scale * log2(e), or 1 for pre-scaled query rows
+    int n_buckets;
+    const void* table; int table_dtype; int64_t t_sbucket, t_shead;
+    BucketSpec bs;
+};
+hipError_t launch_bwd_dense(const BwdParams& p, int dtype, int D, bool causal, hipStream_t stream);
+
 struct RmsParams {
     const void* x; const void* weight; void* y;
     const void* residual; void* sum_out;                  // optional: normalise x + residual, write the sum (input type)

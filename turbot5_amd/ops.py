@@ -190,16 +190,7 @@ def _strides3(t):
     return (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
 
 
-def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                     return_lse: bool = False, exact_scores: Optional[bool] = None):
-    """FlashAttention forward with the T5 relative-position bias computed inside the kernel.
-
-    q (B,H,M,D); k, v (B,H,N,D), any batch/head/row strides; ``bias`` is the
-    (NUM_BUCKETS, H) table or None.  ``causal`` selects the causal mask and the
-    unidirectional buckets together.  ``sm_scale=None`` means 1/sqrt(D).  Returns
-    a tensor shaped and strided like q (``empty_like``), plus the (B,H,M) fp32
-    log-sum-exp when ``return_lse``.
-    """
+def _dense_forward(q, k, v, bias, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, return_lse, exact_scores):
     _check_inputs(q, k, v)
     B, H, M, D = q.shape
     N = k.shape[2]
@@ -222,6 +213,88 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
         L.check(L.load().t5a_fwd_dense(C.byref(a), _stream(q)))
     _commit_lut(keep, B > 0 and M > 0)
     return (o, lse) if return_lse else o
+
+
+def _dense_backward(q, k, v, bias, o, lse, dout, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, exact_scores):
+    """-> dq, dk, dv, dbias (fp32 (NUM_BUCKETS, H), or None without a table); t5a_bwd_dense"""
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    if D == 128:
+        raise NotImplementedError("the backward kernels cover head_dim 16, 32 and 64")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    q_, k_, v_, o_, g_ = (_kernel_ready(t) for t in (q, k, v, o, dout))
+    dq, dk, dv = torch.empty_like(q_), torch.empty_like(k_), torch.empty_like(v_)
+    dtable = torch.empty((NUM_BUCKETS, H), device=q.device, dtype=torch.float32) if bias is not None else None
+    lib = L.load()
+    ws = torch.empty(max(int(lib.t5a_bwd_workspace_bytes(B, H, M)), 16), device=q.device, dtype=torch.uint8)
+    a = L.T5ADenseBwdArgs()
+    a.q, a.k, a.v, a.o, a.dout, a.lse = (t.data_ptr() for t in (q_, k_, v_, o_, g_, lse))
+    a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    a.dtable = dtable.data_ptr() if dtable is not None else None
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    for name, t in (("q_strides", q_), ("k_strides", k_), ("v_strides", v_), ("o_strides", o_), ("dout_strides", g_),
+                    ("dq_strides", dq), ("dk_strides", dk), ("dv_strides", dv)):
+        setattr(a, name, _strides3(t))
+    a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
+    a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.exact_scores = _exact(exact_scores)
+    b = L.T5ABias()
+    keep = None
+    if bias is not None:
+        table = bias.detach()
+        if table.dtype not in _DTYPES:
+            table = table.float()
+        b.table, b.table_dtype = table.data_ptr(), _DTYPES[table.dtype]
+        b.num_buckets, b.max_distance = NUM_BUCKETS, MAX_DISTANCE
+        b.stride_bucket, b.stride_head = table.stride(0), table.stride(1)
+        keep = table
+    a.bias = b
+    with _on_device(q):
+        L.check(lib.t5a_bwd_dense(C.byref(a), _stream(q)))
+    del keep
+    return dq, dk, dv, dtable
+
+
+class FlashAttentionBias(torch.autograd.Function):
+    """The dense fused-bias forward with its backward (reference fused_bias_attention.py:821-873): gradients for q,
+    k, v and the (NUM_BUCKETS, H) table."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, bias, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, exact_scores):
+        o, lse = _dense_forward(q, k, v, bias, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, True, exact_scores)
+        ctx.save_for_backward(q, k, v, o, lse, *(() if bias is None else (bias,)))
+        ctx.has_bias = bias is not None
+        ctx.args = (bool(causal), sm_scale, NUM_BUCKETS, MAX_DISTANCE, exact_scores)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors[:5]
+        bias = ctx.saved_tensors[5] if ctx.has_bias else None
+        causal, sm_scale, nb, md, exact = ctx.args
+        dq, dk, dv, dtable = _dense_backward(q, k, v, bias, o, lse, dout, causal, sm_scale, nb, md, exact)
+        dbias = dtable.to(bias.dtype) if bias is not None and ctx.needs_input_grad[3] else None
+        return dq, dk, dv, dbias, None, None, None, None, None
+
+
+def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
+                                     return_lse: bool = False, exact_scores: Optional[bool] = None):
+    """FlashAttention forward with the T5 relative-position bias computed inside the kernel.
+
+    q (B,H,M,D); k, v (B,H,N,D), any batch/head/row strides; ``bias`` is the
+    (NUM_BUCKETS, H) table or None.  ``causal`` selects the causal mask and the
+    unidirectional buckets together.  ``sm_scale=None`` means 1/sqrt(D).  Returns
+    a tensor shaped and strided like q (``empty_like``), plus the (B,H,M) fp32
+    log-sum-exp when ``return_lse``.  Differentiable in q, k, v and the table (head_dim up to 64), as the
+    reference's autograd function is (fused_bias_attention.py:821-873).
+    """
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (q, k, v, bias))
+    if needs_grad:
+        o, lse = FlashAttentionBias.apply(q, k, v, bias, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, exact_scores)
+        return (o, lse) if return_lse else o
+    return _dense_forward(q, k, v, bias, causal, sm_scale, NUM_BUCKETS, MAX_DISTANCE, return_lse, exact_scores)
 
 
 PLAN_MIN_ITEMS = 3072          # (q tiles x heads) from which a launch plan is built for a single call
