@@ -106,7 +106,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 114
+#define T5A_ABI_VERSION 115
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -208,6 +208,31 @@ typedef struct t5a_varlen_args {
 } t5a_varlen_args;
 int64_t t5a_varlen_workspace_bytes(int32_t B, int32_t H, int32_t total_q);
 int t5a_fwd_varlen(const t5a_varlen_args* args, t5a_stream_t stream);
+
+/*
+ * Backward of t5a_fwd_varlen: dq (total_q,H,D), dk and dv (total_k,H,D), strides {row, head}, and the table
+ * gradient as in t5a_bwd_dense.  Replaces the backward of the reference's packed autograd function
+ * (src/turbot5/ops/varlen_fused_bias_attn.py:407-800, :839-868).  cu_seqlens, seq_lens, causal, sm_scale,
+ * exact_scores and bias as in the forward call; o and lse (total_q, H) are what it returned.  Rows between
+ * cu[b] + seq_lens[b] and cu[b+1] (padding) are not written.  max_seqlen_q / max_seqlen_k size the launch grid:
+ * a longer sequence would lose rows.  workspace: t5a_bwd_varlen_workspace_bytes(total_q, H) bytes.
+ */
+typedef struct t5a_varlen_bwd_args {
+    const void* q; const void* k; const void* v; const void* o; const void* dout; const float* lse;
+    void* dq; void* dk; void* dv; float* dtable;
+    void* workspace; int64_t workspace_bytes;
+    int64_t q_strides[2]; int64_t k_strides[2]; int64_t v_strides[2]; int64_t o_strides[2]; int64_t dout_strides[2];
+    int64_t dq_strides[2]; int64_t dk_strides[2]; int64_t dv_strides[2];
+    const int32_t* cu_seqlens_q; const int32_t* cu_seqlens_k;
+    const int32_t* seq_lens_q; const int32_t* seq_lens_k;
+    int32_t dtype; int32_t B; int32_t H; int32_t D;
+    int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
+    int32_t causal; float sm_scale;
+    int32_t exact_scores; int32_t reserved;
+    t5a_bias bias;
+} t5a_varlen_bwd_args;
+int64_t t5a_bwd_varlen_workspace_bytes(int32_t total_q, int32_t H);
+int t5a_bwd_varlen(const t5a_varlen_bwd_args* args, t5a_stream_t stream);
 
 /*
  * Sparse encoder self-attention as tile skipping (no bias/mask tensor, no

@@ -168,3 +168,106 @@ def test_module_trains_through_the_fused_attention(gpu_device):
     out.square().sum().backward()
     for n, p in mod.named_parameters():
         check(n, p.grad, sd[n].grad, 2e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_packed_gradients_match_autograd_through_the_oracle(gpu_device, dtype, causal):
+    """Backward of the packed forward (t5a_bwd_varlen; reference varlen_fused_bias_attn.py:407-868): every sequence of
+    the batch against autograd through the oracle's dense attention on that sequence alone; the table's gradient is
+    the sum over the sequences."""
+    from turbot5_amd import ops
+    H, D = 3, 64
+    lens = [200, 1, 129, 64, 333]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    total = int(cu[-1])
+    q, k, v = (rnd(total, H, D, seed=40 + i, dtype=dtype) for i in range(3))
+    table = rnd(32, H, seed=43, scale=1.0)
+    dout = rnd(total, H, D, seed=44, scale=1.0, dtype=dtype)
+    wq, wk, wv = (torch.zeros(total, H, D) for _ in range(3))
+    wt = torch.zeros(32, H)
+    for b, n in enumerate(lens):
+        s, e = int(cu[b]), int(cu[b + 1])
+        _, gq, gk, gv, gt = oracle_grads(*(t[s:e].transpose(0, 1)[None] for t in (q, k, v)), table,
+                                         dout[s:e].transpose(0, 1)[None], causal, 1.0)
+        wq[s:e], wk[s:e], wv[s:e] = (g[0].transpose(0, 1) for g in (gq, gk, gv))
+        wt += gt
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    dcu = cu.to(gpu_device)
+    out = ops.flash_attention_with_fusing_bias_varlen(dq, dk, dv, dt, dcu, dcu, max(lens), max(lens), causal=causal, sm_scale=1.0)
+    out.backward(dout.to(gpu_device))
+    tol = TOL[dtype]
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv), ("dtable", dt.grad, wt)):
+        check(name, g, w, tol)
+
+
+def test_packed_gradients_of_a_padded_batch_in_place(gpu_device):
+    """A right-padded (B, L) batch run in place (cu = multiples of L, seq_lens = the lengths), keys longer than the
+    queries in one call (cached decoding shape): padding rows get zero gradients, the rest matches the oracle."""
+    from turbot5_amd import ops
+    B, L, H, D = 3, 160, 2, 64
+    lens = torch.tensor([160, 37, 100], dtype=torch.int32)
+    q, k, v = (rnd(B * L, H, D, seed=50 + i) for i in range(3))
+    table = rnd(32, H, seed=53, scale=1.0)
+    dout = rnd(B * L, H, D, seed=54, scale=1.0)
+    cu = torch.arange(0, (B + 1) * L, L, dtype=torch.int32)
+    wq, wk, wv = (torch.zeros(B * L, H, D) for _ in range(3))
+    wt = torch.zeros(32, H)
+    for b in range(B):
+        s, e = b * L, b * L + int(lens[b])
+        _, gq, gk, gv, gt = oracle_grads(*(t[s:e].transpose(0, 1)[None] for t in (q, k, v)), table,
+                                         dout[s:e].transpose(0, 1)[None], True, 1.0)
+        wq[s:e], wk[s:e], wv[s:e] = (g[0].transpose(0, 1) for g in (gq, gk, gv))
+        wt += gt
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    out = ops.flash_attention_with_fusing_bias_varlen(dq, dk, dv, dt, cu.to(gpu_device), cu.to(gpu_device), L, L, causal=True,
+                                                      sm_scale=1.0, seq_lens_q=lens.to(gpu_device), seq_lens_k=lens.to(gpu_device))
+    out.backward(dout.to(gpu_device))
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv), ("dtable", dt.grad, wt)):
+        assert torch.isfinite(g).all()
+        check(name, g, w, 1e-4)
+    pad = torch.ones(B * L, dtype=torch.bool)
+    for b in range(B):
+        pad[b * L:b * L + int(lens[b])] = False
+    assert (dq.grad.cpu()[pad] == 0).all() and (dk.grad.cpu()[pad] == 0).all() and (dv.grad.cpu()[pad] == 0).all()
+
+
+def test_encoder_stack_trains_and_forward_only_ops_say_so(gpu_device):
+    """A flash encoder in training mode: the loss's gradients reach every parameter (embedding, norms, projections,
+    the bias table of layer 0) and match the oracle's stack differentiated by autograd.  The sparse patterns have no
+    backward kernel and refuse to be differentiated instead of dropping the graph silently."""
+    from oracle import t5_model as OM
+    from turbot5_amd import T5Config, T5EncoderModel, ops
+    # (a smooth feed-forward activation: a ReLU gate that flips between the host's and the device's rounding of a
+    # pre-activation near zero moves a weight gradient by a whole term)
+    cfg = T5Config(vocab_size=64, d_model=128, d_kv=64, d_ff=256, num_layers=2, num_heads=2, dropout_rate=0.0,
+                   attention_type="flash", feed_forward_proj="gated-gelu")
+    torch.manual_seed(5)
+    m = T5EncoderModel(cfg)
+    with torch.no_grad():    # T5's initialisation makes the scores tiny (uniform attention, vanishing q / k gradients)
+        for n, prm in m.named_parameters():
+            if n.endswith(("SelfAttention.q.weight", "SelfAttention.k.weight")):
+                prm.mul_(8.0)
+            if "relative_attention_bias" in n:
+                prm.copy_(torch.randn_like(prm))
+    ids = torch.randint(0, 64, (2, 140), generator=torch.Generator().manual_seed(6))
+    sd = {n: p.detach().clone().requires_grad_(True) for n, p in m.state_dict().items()}
+    # (a loss that the final norm does not make constant: a fixed random functional of the output)
+    r = rnd(2, 140, 128, seed=61, scale=1.0)
+    (OM.encoder_forward(sd, cfg, ids, None, "basic") * r).sum().backward()
+    m = m.to(gpu_device).train()
+    (m(ids.to(gpu_device)) * r.to(gpu_device)).sum().backward()
+    seen = 0
+    for n, p in m.named_parameters():
+        assert p.grad is not None, n
+        if sd[n].grad is not None:
+            # (end to end through two layers of fp32 GEMMs and norms that sum in another order than the host's: the
+            # attention op itself is held to 1e-4 above)
+            check(n, p.grad, sd[n].grad, 3e-3)
+            seen += 1
+    assert seen >= 10
+    q = rnd(1, 2, 256, 64, seed=60).to(gpu_device).requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        ops.local_attention_with_fusing_bias(q, q, q, None, 64)
+    with torch.no_grad():
+        ops.local_attention_with_fusing_bias(q, q, q, None, 64)

@@ -13,13 +13,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 114   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 115   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 SCORES_DEFAULT, SCORES_EXACT, SCORES_PRESCALED = 0, 1, 2   # the exact_scores field
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
-    "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_bwd_dense", "t5a_bwd_workspace_bytes", "t5a_fwd_varlen",
+    "t5a_version", "t5a_last_error", "t5a_bucket_lut", "t5a_fwd_dense", "t5a_bwd_dense", "t5a_bwd_workspace_bytes", "t5a_bwd_varlen", "t5a_bwd_varlen_workspace_bytes", "t5a_fwd_varlen",
     "t5a_varlen_workspace_bytes", "t5a_bias_lut_bytes", "t5a_bias_lut_bytes_windowed",
     "t5a_fwd_sparse", "t5a_sparse_launch_plan", "t5a_sparse_workspace_bytes", "t5a_sparse_key_bits_words", "t5a_splitk_workspace_bytes", "t5a_fwd_splitk", "t5a_fwd_splitk_static",
     "t5a_rmsnorm",
@@ -68,6 +68,22 @@ class T5AVarlenArgs(C.Structure):
                 ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32),
                 ("max_seqlen_k", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
                 ("workspace_ready", C.c_int32), ("exact_scores", C.c_int32),
+                ("bias", T5ABias)]
+
+
+class T5AVarlenBwdArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("dout", C.c_void_p),
+                ("lse", C.c_void_p), ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p), ("dtable", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64),
+                ("q_strides", C.c_int64 * 2), ("k_strides", C.c_int64 * 2), ("v_strides", C.c_int64 * 2),
+                ("o_strides", C.c_int64 * 2), ("dout_strides", C.c_int64 * 2),
+                ("dq_strides", C.c_int64 * 2), ("dk_strides", C.c_int64 * 2), ("dv_strides", C.c_int64 * 2),
+                ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
+                ("seq_lens_q", C.c_void_p), ("seq_lens_k", C.c_void_p),
+                ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
+                ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32), ("max_seqlen_k", C.c_int32),
+                ("causal", C.c_int32), ("sm_scale", C.c_float),
+                ("exact_scores", C.c_int32), ("reserved", C.c_int32),
                 ("bias", T5ABias)]
 
 
@@ -137,6 +153,7 @@ def load() -> C.CDLL:
         lib.t5a_bucket_lut.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32)]
         lib.t5a_bucket_lut.restype = C.c_int
         for name, typ in (("t5a_fwd_dense", T5ADenseArgs), ("t5a_bwd_dense", T5ADenseBwdArgs), ("t5a_fwd_varlen", T5AVarlenArgs),
+                          ("t5a_bwd_varlen", T5AVarlenBwdArgs),
                           ("t5a_fwd_sparse", T5ASparseArgs), ("t5a_fwd_splitk", T5ASplitKArgs),
                           ("t5a_fwd_splitk_static", T5ASplitKArgs)):
             fn = getattr(lib, name)
@@ -144,6 +161,8 @@ def load() -> C.CDLL:
             fn.restype = C.c_int
         lib.t5a_bwd_workspace_bytes.argtypes = [C.c_int32] * 3
         lib.t5a_bwd_workspace_bytes.restype = C.c_int64
+        lib.t5a_bwd_varlen_workspace_bytes.argtypes = [C.c_int32] * 2
+        lib.t5a_bwd_varlen_workspace_bytes.restype = C.c_int64
         lib.t5a_splitk_workspace_bytes.argtypes = [C.c_int32] * 5
         lib.t5a_splitk_workspace_bytes.restype = C.c_int64
         lib.t5a_rmsnorm.argtypes = [C.POINTER(T5ARmsNormArgs), C.c_void_p]

@@ -49,7 +49,9 @@ class T5LayerNorm(nn.Module):
         """On a ROCm device: the fused HIP kernel (the reference switches to its Triton kernel there,
         modules.py:61-66).  Host tensors take the reference's eager formula (modules.py:51-59).
         ``group`` > 1 norms the sums of ``group`` consecutive rows of each sequence (side tokens)."""
-        if x.is_cuda:
+        # (the kernel has no backward: a module in training mode that is being differentiated takes the eager formula)
+        differentiated = self.training and torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad)
+        if x.is_cuda and not (differentiated and seq_lens is None and key_bits is None):
             from .ops import rms_norm
             return rms_norm(x, self.weight, self.eps, group, seq_lens=seq_lens, seq_starts=seq_starts,
                             key_bits=key_bits, group_counts=group_counts)
@@ -72,7 +74,9 @@ class T5LayerNorm(nn.Module):
         ROCm device.  ``residual`` None: ``(x, norm(x))``."""
         if residual is None:
             return x, self.forward(x)
-        if x.is_cuda and residual.dtype == x.dtype and not (torch.is_grad_enabled() and (x.requires_grad or residual.requires_grad)):
+        differentiated = torch.is_grad_enabled() and (x.requires_grad or residual.requires_grad or
+                                                      (self.training and self.weight.requires_grad))
+        if x.is_cuda and residual.dtype == x.dtype and not differentiated:
             from .ops import rms_norm
             return rms_norm(x, self.weight, self.eps, 1, residual)
         total = x + residual

@@ -360,6 +360,65 @@ int t5a_bwd_dense(const t5a_dense_bwd_args* a, t5a_stream_t stream) {
     return finish(launch_bwd_dense(p, a->dtype, a->D, a->causal != 0, (hipStream_t)stream), "t5a_bwd_dense");
 }
 
+int64_t t5a_bwd_varlen_workspace_bytes(int32_t total_q, int32_t H) {
+    if (total_q < 0 || H < 0) return -1;
+    return 2 * (int64_t)total_q * H * (int64_t)sizeof(float);
+}
+
+int t5a_bwd_varlen(const t5a_varlen_bwd_args* a, t5a_stream_t stream) {
+    if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
+    int rc = check_common(a->dtype, a->D);
+    if (rc) return rc;
+    if (a->D == 128) return fail(T5A_ERR_HEAD_DIM, "the backward kernels hold a row's head_dim in registers: head_dim 16, 32 or 64");
+    const int unit = a->dtype == T5A_F32 ? 4 : 8;
+    if (a->B < 0 || a->H <= 0 || a->total_q < 0 || a->total_k < 0 || a->max_seqlen_q < 0 || a->max_seqlen_k < 0)
+        return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d total_q=%d total_k=%d", a->B, a->H, a->total_q, a->total_k);
+    if (a->B == 0 || (a->total_q == 0 && a->total_k == 0)) return T5A_OK;
+    if (a->cu_seqlens_q == nullptr || a->cu_seqlens_k == nullptr) return fail(T5A_ERR_NULL, "cu_seqlens is NULL");
+    if (a->total_q == 0 || a->total_k == 0)
+        return fail(T5A_ERR_SHAPE, "t5a_bwd_varlen needs query rows and keys (total_q=%d total_k=%d)", a->total_q, a->total_k);
+    struct { const char* name; const void* ptr; const int64_t* st; } ts[] = {
+        {"q", a->q, a->q_strides}, {"o", a->o, a->o_strides}, {"dout", a->dout, a->dout_strides}, {"dq", a->dq, a->dq_strides},
+        {"k", a->k, a->k_strides}, {"v", a->v, a->v_strides}, {"dk", a->dk, a->dk_strides}, {"dv", a->dv, a->dv_strides}};
+    for (auto& t : ts)
+        if ((rc = check_tensor(t.name, t.ptr, t.st, 2, unit))) return rc;
+    if (a->lse == nullptr) return fail(T5A_ERR_NULL, "lse is NULL");
+    const int64_t need = t5a_bwd_varlen_workspace_bytes(a->total_q, a->H);
+    if (a->workspace == nullptr || a->workspace_bytes < need)
+        return fail(T5A_ERR_WORKSPACE, "t5a_bwd_varlen: workspace of %lld bytes needed, %lld given", (long long)need, (long long)a->workspace_bytes);
+    if (!aligned16(a->workspace)) return fail(T5A_ERR_STRIDE, "workspace is not 16-byte aligned");
+    if ((int64_t)a->B > 65535 || (int64_t)a->H > 65535) return fail(T5A_ERR_SHAPE, "B or H too large for the launch grid");
+    BwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.dout = a->dout; p.lse = a->lse;
+    p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
+    p.q_sr = a->q_strides[0]; p.q_sh = a->q_strides[1];
+    p.k_sr = a->k_strides[0]; p.k_sh = a->k_strides[1];
+    p.v_sr = a->v_strides[0]; p.v_sh = a->v_strides[1];
+    p.o_sr = a->o_strides[0]; p.o_sh = a->o_strides[1];
+    p.do_sr = a->dout_strides[0]; p.do_sh = a->dout_strides[1];
+    p.dq_sr = a->dq_strides[0]; p.dq_sh = a->dq_strides[1];
+    p.dk_sr = a->dk_strides[0]; p.dk_sh = a->dk_strides[1];
+    p.dv_sr = a->dv_strides[0]; p.dv_sh = a->dv_strides[1];
+    p.B = a->B; p.H = a->H; p.M = a->max_seqlen_q; p.N = a->max_seqlen_k;
+    p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k; p.len_q = a->seq_lens_q; p.len_k = a->seq_lens_k;
+    p.total_q = a->total_q;
+    FwdParams f;
+    memset(&f, 0, sizeof(f));
+    if ((rc = score_mode(a->exact_scores, a->sm_scale, &f))) return rc;
+    p.c1 = f.c1;
+    if ((rc = fill_bias(a->bias, a->causal == 0, &f))) return rc;
+    p.table = f.table; p.table_dtype = f.table_dtype; p.t_sbucket = f.t_sbucket; p.t_shead = f.t_shead; p.bs = f.bs;
+    p.n_buckets = a->bias.table != nullptr ? a->bias.num_buckets : 0;
+    if (a->bias.table != nullptr && a->dtable == nullptr) return fail(T5A_ERR_NULL, "dtable is NULL (the forward had a bias table)");
+    if (p.n_buckets > 4 * kMaxThresholds) return fail(T5A_ERR_BUCKETS, "num_buckets=%d too large for the backward", p.n_buckets);
+    p.dtable = a->bias.table != nullptr ? a->dtable : nullptr;
+    if (p.M == 0 || p.N == 0) return fail(T5A_ERR_SHAPE, "max_seqlen_q and max_seqlen_k must be positive");
+    p.delta = reinterpret_cast<float*>(a->workspace);
+    p.lse2 = p.delta + (int64_t)a->total_q * a->H;
+    return finish(launch_bwd_dense(p, a->dtype, a->D, a->causal != 0, (hipStream_t)stream), "t5a_bwd_varlen");
+}
+
 // Entries per XCD of a packed batch's launch plan: twice the mean, so that slices of equal work but
 // unequal item counts fit (a slice that still outgrows it spills into the others' free slots).
 static int plan_slots(int64_t items_bound) { return (int)(2 * ((items_bound + 7) / 8)); }

@@ -20,6 +20,8 @@
 //                     swapped (query rows from LDS; log-sum-exp and delta of the 64 queries staged in LDS):
 //                     dV^T += dO^T P, dK^T += Q^T dS.
 //
+// With cu_seqlens the same kernels run a packed batch (varlen_fused_bias_attn.py:407-800): a workgroup looks up its
+// sequence's first row and length and works on that sequence; the grid is sized for the longest one.
 // Scores use the key position j and the query position i + N - M, as the forward does; rows whose log-sum-exp is
 // -inf (no visible key) have no gradient.  Rows and keys past the end of a tensor are read as zeros and masked.
 #include "lut_device.h"
@@ -60,19 +62,31 @@ template <typename T> __device__ __forceinline__ void store4(T* p, f32x4 x) {
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const BwdParams p) {
-    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;     // (b, h, i) flattened
-    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    // dense: row = (b, h, i) flattened, statistics (B,H,M); packed: row = (token, h) flattened, statistics (total_q, H)
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool packed = p.cu_q != nullptr;
+    const int64_t rows = packed ? (int64_t)p.total_q * p.H : (int64_t)p.B * p.H * p.M;
     // the table gradient is accumulated with atomics by the dq kernel: clear it here, ahead of that launch
     if (p.dtable != nullptr) {
         const int64_t n = (int64_t)p.n_buckets * p.H;
         for (int64_t x = row; x < n; x += (int64_t)gridDim.x * 256) p.dtable[x] = 0.f;
     }
     if (row >= rows) return;
-    const int i = (int)(row % p.M);
-    const int64_t bh = row / p.M;
-    const int h = (int)(bh % p.H), b = (int)(bh / p.H);
-    const T* o = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)i * p.o_sr;
-    const T* g = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + (int64_t)i * p.do_sr;
+    int64_t o_off, g_off;
+    if (packed) {
+        const int64_t tok = row / p.H;
+        const int h = (int)(row - tok * p.H);
+        o_off = tok * p.o_sr + (int64_t)h * p.o_sh;
+        g_off = tok * p.do_sr + (int64_t)h * p.do_sh;
+    } else {
+        const int i = (int)(row % p.M);
+        const int64_t bh = row / p.M;
+        const int h = (int)(bh % p.H), b = (int)(bh / p.H);
+        o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)i * p.o_sr;
+        g_off = (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + (int64_t)i * p.do_sr;
+    }
+    const T* o = reinterpret_cast<const T*>(p.o) + o_off;
+    const T* g = reinterpret_cast<const T*>(p.dout) + g_off;
     float acc = 0.f;
 #pragma unroll
     for (int c = 0; c < D / 4; ++c) {
@@ -102,16 +116,28 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
     const int h = blockIdx.y, b = blockIdx.z;
     const int own_base = blockIdx.x * kBwdOwn;
     const int own_row = own_base + wave * 32 + lr;
-    const int n_own = KV ? p.N : p.M, n_other = KV ? p.M : p.N;
-    const int P = p.N - p.M;                       // query i sits at key position i + P
+    // packed batch: sequence b is the rows [cu[b], cu[b] + len) of the (total, H, D) tensors (len from seq_lens when
+    // given, else up to cu[b + 1]); the batch strides are 0 and everything below works on that sequence
+    int M = p.M, N = p.N;
+    int64_t q_first = 0, k_first = 0;
+    if (p.cu_q != nullptr) {
+        q_first = p.cu_q[b]; k_first = p.cu_k[b];
+        M = p.len_q != nullptr ? p.len_q[b] : p.cu_q[b + 1] - (int)q_first;
+        N = p.len_k != nullptr ? p.len_k[b] : p.cu_k[b + 1] - (int)k_first;
+        if (own_base >= (KV ? N : M)) return;     // (the grid is sized for the longest sequence)
+    }
+    const int n_own = KV ? N : M, n_other = KV ? M : N;
+    const int P = N - M;                           // query i sits at key position i + P
     const bool has_bias = p.table != nullptr;
     const int sat = has_bias ? p.bs.sat : 0;
 
-    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
-    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
-    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
-    const T* gp = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.do_sb + (int64_t)h * p.do_sh;
-    const int64_t stat_base = ((int64_t)b * p.H + h) * p.M;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh + q_first * p.q_sr;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh + k_first * p.k_sr;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)h * p.v_sh + k_first * p.v_sr;
+    const T* gp = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + q_first * p.do_sr;
+    // statistics of query i: index stat_base + i * stat_sr
+    const int64_t stat_sr = p.cu_q != nullptr ? p.H : 1;
+    const int64_t stat_base = p.cu_q != nullptr ? q_first * p.H + h : ((int64_t)b * p.H + h) * p.M;
 
     // bias (and bucket) per clamped distance
     if (has_bias) {
@@ -139,7 +165,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
         }
     }
     float lse2_own = INFINITY, delta_own = 0.f;
-    if (!KV && own_ok) { lse2_own = p.lse2[stat_base + own_row]; delta_own = p.delta[stat_base + own_row]; }
+    if (!KV && own_ok) { lse2_own = p.lse2[stat_base + own_row * stat_sr]; delta_own = p.delta[stat_base + own_row * stat_sr]; }
 
     // tiles of the other kind that can hold a visible pair
     int t_lo = 0, t_hi = (n_other + kBwdOther - 1) / kBwdOther;
@@ -175,7 +201,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
             if (KV && tid < 2 * kBwdOther) {
                 const int row = tid & (kBwdOther - 1);
                 float val = tid < kBwdOther ? INFINITY : 0.f;
-                if (o0 + row < n_other) val = tid < kBwdOther ? p.lse2[stat_base + o0 + row] : p.delta[stat_base + o0 + row];
+                if (o0 + row < n_other)
+                    val = tid < kBwdOther ? p.lse2[stat_base + (o0 + row) * stat_sr] : p.delta[stat_base + (o0 + row) * stat_sr];
                 rowstat[tid] = val;
             }
         }
@@ -209,7 +236,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
                 const int ol = 32 * nt + 8 * (r >> 2) + 4 * hh + (r & 3);   // row of the other kind inside the tile
                 const int i = KV ? o0 + ol : own_row, j = KV ? own_row : o0 + ol;
                 const int rel = j - (i + P);
-                const bool valid = i < p.M && j < p.N && (!CAUSAL || rel <= 0);
+                const bool valid = i < M && j < N && (!CAUSAL || rel <= 0);
                 const int x = min(max(rel, -sat), sat) + sat;
                 const float bias2 = has_bias ? lut_bias[x] : 0.f;
                 const float l2 = KV ? rowstat[ol] : lse2_own;
@@ -245,9 +272,9 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
     // rows: lane (lr, hh) holds, for its own row, elements 32 dt + 8 g + 4 hh .. + 3 of the transposed gradients
     const float scale = p.c1 * 0.6931471805599453f;     // d score / d (q . k), natural units
     if (own_ok) {
-        T* oa = KV ? reinterpret_cast<T*>(p.dk) + (int64_t)b * p.dk_sb + (int64_t)h * p.dk_sh + (int64_t)own_row * p.dk_sr
-                   : reinterpret_cast<T*>(p.dq) + (int64_t)b * p.dq_sb + (int64_t)h * p.dq_sh + (int64_t)own_row * p.dq_sr;
-        T* ob = KV ? reinterpret_cast<T*>(p.dv) + (int64_t)b * p.dv_sb + (int64_t)h * p.dv_sh + (int64_t)own_row * p.dv_sr : nullptr;
+        T* oa = KV ? reinterpret_cast<T*>(p.dk) + (int64_t)b * p.dk_sb + (int64_t)h * p.dk_sh + (k_first + own_row) * p.dk_sr
+                   : reinterpret_cast<T*>(p.dq) + (int64_t)b * p.dq_sb + (int64_t)h * p.dq_sh + (q_first + own_row) * p.dq_sr;
+        T* ob = KV ? reinterpret_cast<T*>(p.dv) + (int64_t)b * p.dv_sb + (int64_t)h * p.dv_sh + (k_first + own_row) * p.dv_sr : nullptr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -282,7 +309,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd_kernel(const BwdParams p) 
 
 template <typename T, int D>
 hipError_t launch_bwd_d(const BwdParams& p, bool causal, hipStream_t stream) {
-    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    const int64_t rows = p.cu_q != nullptr ? (int64_t)p.total_q * p.H : (int64_t)p.B * p.H * p.M;
     hipLaunchKernelGGL((bwd_rows_kernel<T, D>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -134,7 +134,10 @@ struct BwdParams {
     float* delta; float* lse2;        // workspace, (B,H,M) each
     int64_t q_sb, q_sh, q_sr, k_sb, k_sh, k_sr, v_sb, v_sh, v_sr, o_sb, o_sh, o_sr, do_sb, do_sh, do_sr;
     int64_t dq_sb, dq_sh, dq_sr, dk_sb, dk_sh, dk_sr, dv_sb, dv_sh, dv_sr;
-    int B, H, M, N;
+    int B, H, M, N;                   // packed: M, N are the longest sequence's lengths
+    // packed batch (optional): (B+1) offsets and optional lengths, as in the forward; tensors are (total, H, D),
+    // the statistics (total_q, H)
+    const int32_t* cu_q; const int32_t* cu_k; const int32_t* len_q; const int32_t* len_k; int total_q;
     float c1;                         // base-2 score factor: sm_scale * log2(e), or 1 for pre-scaled query rows
     int n_buckets;
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;

@@ -74,6 +74,14 @@ def _check_inputs(q, k, v):
     assert Dk in {16, 32, 64, 128}              # fused_bias_attention.py:828
 
 
+def _forward_only(what: str, *tensors):
+    """The sparse patterns, split-K decoding and the RMS norm kernel have no backward: say so instead of returning
+    a result that silently carries no graph."""
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise NotImplementedError(f"{what} is forward only (no backward kernel); run it under torch.no_grad() or "
+                                  "use attention_type='flash', whose kernels have one")
+
+
 def _unit(t: torch.Tensor) -> int:
     return 4 if t.dtype == torch.float32 else 8
 
@@ -331,25 +339,8 @@ class LaunchPlan:
         self.key, self.tensors = key, tensors
 
 
-def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                                            causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
-                                            return_lse: bool = False, seq_lens_q=None, seq_lens_k=None,
-                                            launch_plan: bool = True, exact_scores: Optional[bool] = None):
-    """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
-
-    Positions restart at 0 in every sequence.  No host synchronisation: the
-    work list is derived on the device from ``cu_seqlens``.
-
-    ``seq_lens_q`` / ``seq_lens_k`` (optional int32 device tensors of B lengths): sequence b is rows
-    [cu[b], cu[b] + lens[b]); the rows up to cu[b+1] are padding, never read and left ZERO in the
-    output.  A right-padded (B, L, H, D) batch runs in place this way, viewed as (B*L, H, D) with
-    cu = arange(B+1) * L and lens = mask.sum(-1): no gathers, no scatter.
-
-    ``launch_plan``: True (default) lets larger launches first build, on the device, per-XCD item
-    lists of equal work from ``cu_seqlens`` (a small workspace is taken from torch's allocator);
-    False never does, ``"always"`` does whatever the size.  A ``LaunchPlan`` object keeps the plan
-    for later calls over the same batch.  The results do not depend on any of this.
-    """
+def _varlen_forward(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale, NUM_BUCKETS,
+                    MAX_DISTANCE, return_lse, seq_lens_q, seq_lens_k, launch_plan, exact_scores):
     _check_inputs(q, k, v)
     total_q, H, D = q.shape
     total_k = k.shape[0]
@@ -418,6 +409,112 @@ def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seql
     return (o, lse) if return_lse else o
 
 
+def _varlen_backward(q, k, v, bias, o, lse, dout, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale,
+                     NUM_BUCKETS, MAX_DISTANCE, seq_lens_q, seq_lens_k, exact_scores):
+    """-> dq, dk, dv, dbias (fp32 (NUM_BUCKETS, H) or None); t5a_bwd_varlen"""
+    total_q, H, D = q.shape
+    if D == 128:
+        raise NotImplementedError("the backward kernels cover head_dim 16, 32 and 64")
+    B = cu_seqlens_q.numel() - 1
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    cq = cu_seqlens_q.to(device=q.device, dtype=torch.int32).contiguous()
+    ck = cq if cu_seqlens_k is cu_seqlens_q else cu_seqlens_k.to(device=q.device, dtype=torch.int32).contiguous()
+    lens = [t.to(device=q.device, dtype=torch.int32).contiguous() if t is not None else None for t in (seq_lens_q, seq_lens_k)]
+    q_, k_, v_, o_, g_ = (_kernel_ready(t) for t in (q, k, v, o, dout))
+    # rows of padding (between a sequence's length and the next sequence's first row) get no gradient
+    dq = (torch.empty_like if lens[0] is None else torch.zeros_like)(q_)
+    dk = (torch.empty_like if lens[1] is None else torch.zeros_like)(k_)
+    dv = (torch.empty_like if lens[1] is None else torch.zeros_like)(v_)
+    dtable = torch.empty((NUM_BUCKETS, H), device=q.device, dtype=torch.float32) if bias is not None else None
+    lib = L.load()
+    ws = torch.empty(max(int(lib.t5a_bwd_varlen_workspace_bytes(total_q, H)), 16), device=q.device, dtype=torch.uint8)
+    a = L.T5AVarlenBwdArgs()
+    a.q, a.k, a.v, a.o, a.dout, a.lse = (t.data_ptr() for t in (q_, k_, v_, o_, g_, lse))
+    a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    a.dtable = dtable.data_ptr() if dtable is not None else None
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    for name, t in (("q_strides", q_), ("k_strides", k_), ("v_strides", v_), ("o_strides", o_), ("dout_strides", g_),
+                    ("dq_strides", dq), ("dk_strides", dk), ("dv_strides", dv)):
+        setattr(a, name, (C.c_int64 * 2)(t.stride(0), t.stride(1)))
+    a.cu_seqlens_q, a.cu_seqlens_k = cq.data_ptr(), ck.data_ptr()
+    a.seq_lens_q = lens[0].data_ptr() if lens[0] is not None else None
+    a.seq_lens_k = lens[1].data_ptr() if lens[1] is not None else None
+    a.dtype, a.B, a.H, a.D = _dtype_code(q), B, H, D
+    a.total_q, a.total_k = total_q, k.shape[0]
+    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
+    a.exact_scores = _exact(exact_scores)
+    b = L.T5ABias()
+    table = None
+    if bias is not None:
+        table = bias.detach()
+        if table.dtype not in _DTYPES:
+            table = table.float()
+        b.table, b.table_dtype = table.data_ptr(), _DTYPES[table.dtype]
+        b.num_buckets, b.max_distance = NUM_BUCKETS, MAX_DISTANCE
+        b.stride_bucket, b.stride_head = table.stride(0), table.stride(1)
+    a.bias = b
+    with _on_device(q):
+        L.check(lib.t5a_bwd_varlen(C.byref(a), _stream(q)))
+    del table
+    return dq, dk, dv, dtable
+
+
+class FlashAttentionBiasVarlen(torch.autograd.Function):
+    """The packed forward with its backward (reference varlen_fused_bias_attn.py:800-868)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale, NUM_BUCKETS,
+                MAX_DISTANCE, seq_lens_q, seq_lens_k, launch_plan, exact_scores):
+        o, lse = _varlen_forward(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale,
+                                 NUM_BUCKETS, MAX_DISTANCE, True, seq_lens_q, seq_lens_k, launch_plan, exact_scores)
+        ctx.save_for_backward(q, k, v, o, lse, *(() if bias is None else (bias,)))
+        ctx.has_bias = bias is not None
+        ctx.args = (cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, bool(causal), sm_scale, NUM_BUCKETS, MAX_DISTANCE,
+                    seq_lens_q, seq_lens_k, exact_scores)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors[:5]
+        bias = ctx.saved_tensors[5] if ctx.has_bias else None
+        cq, ck, mq, mk, causal, sm_scale, nb, md, lq, lk, exact = ctx.args
+        dq, dk, dv, dtable = _varlen_backward(q, k, v, bias, o, lse, dout, cq, ck, mq, mk, causal, sm_scale, nb, md, lq, lk, exact)
+        dbias = dtable.to(bias.dtype) if bias is not None and ctx.needs_input_grad[3] else None
+        return (dq, dk, dv, dbias) + (None,) * 12
+
+
+def flash_attention_with_fusing_bias_varlen(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                            causal=False, sm_scale=None, NUM_BUCKETS=32, MAX_DISTANCE=128,
+                                            return_lse: bool = False, seq_lens_q=None, seq_lens_k=None,
+                                            launch_plan: bool = True, exact_scores: Optional[bool] = None):
+    """Packed variable-length forward: q (total_q,H,D), k/v (total_k,H,D), cu_seqlens int32 on the device.
+
+    Positions restart at 0 in every sequence.  No host synchronisation: the
+    work list is derived on the device from ``cu_seqlens``.
+
+    ``seq_lens_q`` / ``seq_lens_k`` (optional int32 device tensors of B lengths): sequence b is rows
+    [cu[b], cu[b] + lens[b]); the rows up to cu[b+1] are padding, never read and left ZERO in the
+    output.  A right-padded (B, L, H, D) batch runs in place this way, viewed as (B*L, H, D) with
+    cu = arange(B+1) * L and lens = mask.sum(-1): no gathers, no scatter.
+
+    ``launch_plan``: True (default) lets larger launches first build, on the device, per-XCD item
+    lists of equal work from ``cu_seqlens`` (a small workspace is taken from torch's allocator);
+    False never does, ``"always"`` does whatever the size.  A ``LaunchPlan`` object keeps the plan
+    for later calls over the same batch.  The results do not depend on any of this.
+    """
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (q, k, v, bias))
+    if needs_grad:
+        o, lse = FlashAttentionBiasVarlen.apply(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
+                                                sm_scale, NUM_BUCKETS, MAX_DISTANCE, seq_lens_q, seq_lens_k, launch_plan,
+                                                exact_scores)
+        return (o, lse) if return_lse else o
+    return _varlen_forward(q, k, v, bias, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale,
+                           NUM_BUCKETS, MAX_DISTANCE, return_lse, seq_lens_q, seq_lens_k, launch_plan, exact_scores)
+
+
 KEY_BITS_FRONT = 8   # zero words in front of a sequence's validity bits (kKeyBitsFront of the library)
 
 
@@ -451,6 +548,7 @@ def _sparse(pattern, q, k, v, bias, block_len, aux, side_k=None, side_v=None, sm
             NUM_BUCKETS=32, MAX_DISTANCE=128, key_splits=True, seq_lens=None, exact_scores=None, seq_starts=None,
             key_bits=None, side_counts=None):
     _check_inputs(q, k, v)
+    _forward_only("sparse attention (local, block, transient-global)", q, k, v, bias, side_k, side_v)
     B, H, Lq, D = q.shape
     if side_counts is not None and (pattern != L.PATTERN_TGLOBAL or key_bits is None):
         raise ValueError("side_counts goes with key_bits in the transient-global pattern")
