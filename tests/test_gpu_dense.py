@@ -540,3 +540,55 @@ def test_output_in_token_major_layout_with_guard_rows(gpu_device, dt, D):
     assert (got - want).abs().max().item() <= TOL[dt]
     host = buf.float().cpu()
     assert (host[:, M:] == fill).all() and (host[:, :, H] == fill).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["ramp", "late_outlier", "early_outlier", "huge_everywhere", "tiny_everywhere"])
+def test_running_max_is_raised_from_the_row_sums(gpu_device, dtype, causal, kind):
+    """The dense fast steps at head_dim 64 form no row maximum: a tile's row sum tells whether the running max must
+    be raised, and a rare block then looks the exact maximum up and forms the tile's exponentials again, before the
+    tile reaches the output accumulators.  Scores built to exercise that block:
+      ramp             every key tile scores about 40 above the one before it (base-2 units): a raise in every step
+      late_outlier     one key near the end scores 300 above everything: its exponential overflows fp32 against the
+                       stale maximum, and must never reach the accumulators
+      early_outlier    the same in the first tile: everything later underflows against it
+      huge / tiny      all scores around +400 / -400: no probability may overflow or underflow as a whole
+    Keys are multiples of one direction u, queries carry a unit component along u, so q.k is the key's multiple and
+    exact in the 16-bit types; values are random.  Against the oracle in fp32 on the same inputs."""
+    from turbot5_amd.ops import flash_attention_with_fusing_bias
+    B, H, L, D = 1, 2, 1024, 64
+    g = torch.Generator().manual_seed(77)
+    u = torch.zeros(D)
+    u[0] = 1.0
+    q = 0.05 * torch.randn(B, H, L, D, generator=g)
+    q[..., 0] = 1.0                                     # q . (c u) = c
+    j = torch.arange(L, dtype=torch.float32)
+    if kind == "ramp":
+        c = 28.0 * (j // 64)                            # nats: about 40 per tile in base-2 units
+    elif kind == "late_outlier":
+        c = torch.zeros(L)
+        c[L - 37] = 208.0
+    elif kind == "early_outlier":
+        c = torch.zeros(L)
+        c[5] = 208.0
+    elif kind == "huge_everywhere":
+        c = 280.0 + (j % 7)
+    else:
+        c = -280.0 - (j % 7)
+    if dtype == torch.float16:
+        c = c * 0.5                                     # (fp16 holds the keys' multiples up to 65504; keep them exact)
+    k = (c[:, None] * u[None, :]).expand(B, H, L, D).clone()
+    k[..., 1:] = 0.05 * torch.randn(B, H, L, D - 1, generator=g)
+    v = torch.randn(B, H, L, D, generator=g)
+    q, k, v = (t.to(dtype) for t in (q, k, v))
+    table = torch.randn(32, H, generator=g)
+    want = O.dense_attention(q, k, v, table, causal, 1.0)
+    for exact in (None, True):
+        got = flash_attention_with_fusing_bias(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), table.to(gpu_device),
+                                               causal=causal, sm_scale=1.0, exact_scores=exact).float().cpu()
+        assert torch.isfinite(got).all(), (kind, exact)
+        # (scores this large make one key's weight 1: the default mode's extra rounding of Q moves scores of several
+        # hundred by whole units, so it is compared on the kinds whose result does not hang on a single unit)
+        if exact or kind in ("late_outlier", "early_outlier"):
+            assert (got - want).abs().max().item() <= 3e-2, (kind, exact)

@@ -1959,13 +1959,17 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 // stage holds zeros or a tile of the next q tile) and nobody consumes it, so the run may end
                 // exactly there.
                 const int run = plain_run(t);
-                int quads = (t + run >= ntiles ? run : run - 1) >> 2;
-                if (quads > 0) {
+                const int fast = t + run >= ntiles ? run : run - 1;   // steps from here on that can be fast ones
+                int quads = fast >> 2;
+                // dense kinds: two more fast steps behind the groups of four (ring stages 0 and 1), so that the tail of
+                // a short or causal item takes fewer general steps
+                const bool pair = V2 && fast >= 2 && (fast & 3) >= 2;
+                const bool ran_fast = quads > 0 || pair;
+                if (ran_fast) {
                     tc = classify(t);
                     if constexpr (DENSE) { cursor_seek(t + 4, t + 3); fc_until = 0; }
                 }
-                if (quads > 0) T5A_PHASE_START();
-                const bool ran_fast = quads > 0;
+                if (ran_fast) T5A_PHASE_START();
                 if (V2 && ran_fast) dense_enter(sta);
                 while (quads > 0) {
                     fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
@@ -1973,6 +1977,11 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
                     fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
                     --quads; t += 4;
+                }
+                if (pair) {
+                    fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
+                    fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
+                    t += 2;
                 }
                 // (the dense fast steps leave the tile that follows them without its head: the general step wants
                 // it done; its early exponentials are simply formed again there)
