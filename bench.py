@@ -23,7 +23,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                         difference between what the timed launches wrote and that CPU path on row subsets
 
 --leg NAME runs one kernel K times and nothing else, for profiling:
-    dense:BxL[c][:exact|:prescaled]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
+    dense:BxL[c][:exact|:prescaled]  bwd:BxL[c]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
 --leg NAME --timeline does the same with the measurement build of the library (`python -m turbot5_amd.build --trace`)
 and prints where the work items of the last launch spent their shader-clock cycles.
 """
@@ -222,6 +222,17 @@ def extra_workloads(torch, dev, steps, samples):
                 samples.append(dense_sample(torch, f"dense_B{bsz}_L{ln}_{mode}", qref, k, v, table, f(), False, bsz - 1, 2, 34))
         del q, k, v, qs
     out["score_modes"] = modes
+
+    # ---- backward of the dense forward at the headline shape (dq, dk, dv, table gradient; fp32 matrix cores)
+    q, k, v, table = make_inputs(torch, dev, B, H, L, D)
+    o, lse = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0, return_lse=True)
+    gout = torch.randn_like(o)
+    f = lambda: ops._dense_backward(q, k, v, table, o, lse, gout, False, 1.0, 32, 128, None)  # noqa: E731
+    _, ms = time_kernel(torch, f, reps, warm)
+    tf = 10.0 * B * H * D * L * L / (ms * 1e-3) / 1e12
+    out["backward_B16_H12_L1024"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_fp32_mfma_peak": round(tf / PEAK_F32_TFLOPS, 4),
+                                     "note": "three kernels; 2.5 x the forward's FLOPs, fp32 arithmetic whatever the tensors' type"}
+    del q, k, v, o, gout
 
     # ---- head_dim 128 (the T5-3B / 11B head shape): B4 H6 L4096, same FLOPs as the B4 H12 D64 sweep point
     g = torch.Generator().manual_seed(6)
@@ -524,6 +535,18 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
         exact = {None: None, "exact": True, "prescaled": "prescaled"}[mode]
         f = lambda: ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0, exact_scores=exact)  # noqa: E731
         fl = 4.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
+    elif name.startswith("bwd:"):
+        # the backward kernels alone (dq pass, dk / dv pass, row statistics) on saved forward results: 2.5 x the
+        # forward's FLOPs (five products instead of two), all on the fp32 matrix cores
+        shape = name.split(":")[1]
+        causal = shape.endswith("c")
+        b, l = (int(x) for x in shape.rstrip("c").split("x"))
+        q, k, v, table = make_inputs(torch, dev, b, H, l, D, seed=l if (b, l) != (B, L) else 0)
+        o, lse = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0, return_lse=True)
+        g = torch.randn_like(o)
+        f = lambda: ops._dense_backward(q, k, v, table, o, lse, g, causal, 1.0, 32, 128, None)  # noqa: E731
+        fl = 10.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
+        peak = PEAK_F32_TFLOPS
     elif name == "dense_f32_c1":
         # the attention of baseline configuration 1 (T5-small encoder): B4 H8 L512 D64 in fp32, on the fp32 matrix cores
         g = torch.Generator().manual_seed(3)
@@ -617,7 +640,7 @@ def main():
     ap.add_argument("--no-models", action="store_true", help="skip the T5-base model legs (encoder, 100k pass, decoding)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and its checks")
     ap.add_argument("--leg", default=None, metavar="NAME",
-                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
+                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], bwd:BxL[c], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
     ap.add_argument("--timeline", action="store_true",
                     help="with --leg: use the measurement build (libt5attn_trace.so) and print the work items' cycle stamps")
     ap.add_argument("--full", action="store_true", help="accepted for compatibility: the default run is the full one")
