@@ -106,7 +106,7 @@ int64_t t5a_bias_lut_bytes_windowed(int32_t H, int32_t num_buckets, int32_t max_
 
 /* Layout of the argument structs and set of entry points; a binding compares it with t5a_version() before
  * it passes a struct (a stale library would read pointers from the wrong offsets). */
-#define T5A_ABI_VERSION 115
+#define T5A_ABI_VERSION 116
 int t5a_version(void);
 const char* t5a_last_error(void);
 
@@ -147,8 +147,14 @@ int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
  * q, k, v, causal, sm_scale, exact_scores and bias as in the forward call; o and lse are what it returned
  * (lse is required); dout is the gradient of o.  dq (B,H,M,D), dk and dv (B,H,N,D) in the tensors' type, any
  * strides {batch, head, row}; dtable (required when bias.table is set): (num_buckets, H) contiguous fp32, overwritten.
- * head_dim 16, 32 or 64.  All arithmetic is fp32 (fp32 matrix cores) whatever the tensors' type.  The table
- * gradient is summed with floating-point atomics: its last bits depend on the order of the workgroups.
+ * head_dim 16, 32 or 64.  The table gradient is summed with floating-point atomics: its last bits depend on the
+ * order of the workgroups.
+ * Arithmetic of the backward.  fp32 tensors, head_dim 16 and 32, and any call with fp32_math != 0: every product on
+ * the fp32 matrix cores, inputs widened on their way in.  16-bit tensors at head_dim 64 with fp32_math == 0: the
+ * 16-bit matrix cores -- the score and dP products take the inputs as they are, and the probabilities and dS are
+ * rounded to the tensors' type before the products that form dq, dk and dv, as the reference rounds them
+ * (fused_bias_attention.py:575-590); sums, the softmax statistics and the table gradient stay in fp32.  About
+ * five times faster; gradients differ from the fp32 path by the rounding of their own type.
  * workspace: t5a_bwd_workspace_bytes(B, H, M) bytes of 16-byte aligned device memory.
  */
 typedef struct t5a_dense_bwd_args {
@@ -159,7 +165,7 @@ typedef struct t5a_dense_bwd_args {
     int64_t dq_strides[3]; int64_t dk_strides[3]; int64_t dv_strides[3];
     int32_t dtype; int32_t B; int32_t H; int32_t M; int32_t N; int32_t D;
     int32_t causal; float sm_scale;
-    int32_t exact_scores; int32_t reserved;
+    int32_t exact_scores; int32_t fp32_math;   /* fp32_math: see "Arithmetic of the backward" above */
     t5a_bias bias;
 } t5a_dense_bwd_args;
 int64_t t5a_bwd_workspace_bytes(int32_t B, int32_t H, int32_t M);
@@ -228,7 +234,7 @@ typedef struct t5a_varlen_bwd_args {
     int32_t dtype; int32_t B; int32_t H; int32_t D;
     int32_t total_q; int32_t total_k; int32_t max_seqlen_q; int32_t max_seqlen_k;
     int32_t causal; float sm_scale;
-    int32_t exact_scores; int32_t reserved;
+    int32_t exact_scores; int32_t fp32_math;   /* as in t5a_dense_bwd_args */
     t5a_bias bias;
 } t5a_varlen_bwd_args;
 int64_t t5a_bwd_varlen_workspace_bytes(int32_t total_q, int32_t H);

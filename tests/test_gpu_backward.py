@@ -1,7 +1,8 @@
 """Backward of the dense fused-bias forward (t5a_bwd_dense behind ops.FlashAttentionBias) against torch.autograd
 through the oracle's dense attention on the same seeded inputs: dq, dk, dv and the gradient of the
 (num_buckets, H) table.  fp32: 1e-4 relative to the gradient's scale; bf16 / fp16: 2e-2 relative to it (the
-oracle differentiates fp32 math on the rounded inputs; the kernels do the same and round only their results).
+oracle differentiates fp32 math on the rounded inputs; the fp32 kernels do the same and round only their results,
+the 16-bit kernels at head_dim 64 also round the probabilities and dS to the tensors' type, as the reference does).
 Reference: src/turbot5/ops/fused_bias_attention.py:397-873."""
 import ctypes as C
 
@@ -75,6 +76,49 @@ def test_gradients_of_strided_views_without_a_table_and_with_a_scale(gpu_device,
     out.backward(dout.to(gpu_device))
     for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv)):
         check(name, g, w, 1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("M,N", [(1024, 1024), (640, 1152), (1100, 700)])
+def test_16_bit_gradients_over_long_rows(gpu_device, dtype, causal, M, N):
+    """16-bit tensors at head_dim 64 run on the 16-bit matrix cores.  Rows long enough for every kind of tile of
+    both passes: distances saturated on either side of the diagonal (constant bias, table gradient from tile sums),
+    the band around it (bias per distance, table gradient from the sums along the tile's diagonals), tiles cut by
+    the causal mask and by the ends of the tensors, several workgroups per (batch, head)."""
+    from turbot5_amd import ops
+    B, H, D = 1, 2, 64
+    q, k, v = rnd(B, H, M, D, seed=61, dtype=dtype), rnd(B, H, N, D, seed=62, dtype=dtype), rnd(B, H, N, D, seed=63, dtype=dtype)
+    table = rnd(32, H, seed=64, scale=1.0)
+    dout = rnd(B, H, M, D, seed=65, scale=1.0, dtype=dtype)
+    _, wq, wk, wv, wt = oracle_grads(q, k, v, table, dout, causal, 1.0)
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    ops.flash_attention_with_fusing_bias(dq, dk, dv, dt, causal=causal, sm_scale=1.0).backward(dout.to(gpu_device))
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv), ("dtable", dt.grad, wt)):
+        check(name, g, w, TOL[dtype])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_16_bit_gradients_on_the_fp32_matrix_cores_and_of_strided_views(gpu_device, monkeypatch, causal):
+    """fp32_math: the fp32 kernels also for 16-bit tensors at head_dim 64 (they only round their results), so the two
+    paths bracket each other: both within the 16-bit bar of the oracle, the fp32 one within half of it.  On
+    (B, L, H, D) memory viewed as (B, H, L, D), without a table and with the default scale as well."""
+    from turbot5_amd import ops
+    B, H, L, D = 2, 3, 320, 64
+    q, k, v = (rnd(B, L, H, D, seed=70 + i, dtype=torch.bfloat16).transpose(1, 2) for i in range(3))
+    dout = rnd(B, L, H, D, seed=73, scale=1.0, dtype=torch.bfloat16).transpose(1, 2)
+    table = rnd(32, H, seed=74, scale=1.0)
+    for tab, scale in ((table, 1.0), (None, None)):
+        _, wq, wk, wv, wt = oracle_grads(q, k, v, tab, dout, causal, scale)
+        for fp32_math, tol in ((False, 2e-2), (True, 1e-2)):
+            monkeypatch.setattr(ops, "BACKWARD_FP32_MATH", fp32_math)
+            dq, dk, dv = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+            dt = tab.to(gpu_device).requires_grad_(True) if tab is not None else None
+            ops.flash_attention_with_fusing_bias(dq, dk, dv, dt, causal=causal, sm_scale=scale).backward(dout.to(gpu_device))
+            for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv)):
+                check(f"{name} fp32_math={fp32_math}", g, w, tol)
+            if tab is not None:
+                check(f"dtable fp32_math={fp32_math}", dt.grad, wt, tol)
 
 
 def test_gradients_with_prescaled_query_rows(gpu_device):

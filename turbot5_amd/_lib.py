@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libt5attn.so")
 
 T5A_BF16, T5A_F32, T5A_F16 = 0, 1, 2
-ABI_VERSION = 115   # T5A_ABI_VERSION of include/t5attn.h
+ABI_VERSION = 116   # T5A_ABI_VERSION of include/t5attn.h
 PATTERN_LOCAL, PATTERN_BLOCK, PATTERN_TGLOBAL = 1, 2, 3
 SCORES_DEFAULT, SCORES_EXACT, SCORES_PRESCALED = 0, 1, 2   # the exact_scores field
 STATIC_SCRATCH_BYTES = 8 * 1024 * 1024   # T5A_STATIC_SCRATCH_BYTES
@@ -53,7 +53,7 @@ class T5ADenseBwdArgs(C.Structure):
                 ("dq_strides", C.c_int64 * 3), ("dk_strides", C.c_int64 * 3), ("dv_strides", C.c_int64 * 3),
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("M", C.c_int32), ("N", C.c_int32),
                 ("D", C.c_int32), ("causal", C.c_int32), ("sm_scale", C.c_float),
-                ("exact_scores", C.c_int32), ("reserved", C.c_int32),
+                ("exact_scores", C.c_int32), ("fp32_math", C.c_int32),
                 ("bias", T5ABias)]
 
 
@@ -83,7 +83,7 @@ class T5AVarlenBwdArgs(C.Structure):
                 ("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("total_q", C.c_int32), ("total_k", C.c_int32), ("max_seqlen_q", C.c_int32), ("max_seqlen_k", C.c_int32),
                 ("causal", C.c_int32), ("sm_scale", C.c_float),
-                ("exact_scores", C.c_int32), ("reserved", C.c_int32),
+                ("exact_scores", C.c_int32), ("fp32_math", C.c_int32),
                 ("bias", T5ABias)]
 
 

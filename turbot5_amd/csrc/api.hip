@@ -355,6 +355,7 @@ int t5a_bwd_dense(const t5a_dense_bwd_args* a, t5a_stream_t stream) {
             e = hipMemsetAsync(p.dtable, 0, (size_t)p.n_buckets * a->H * sizeof(float), (hipStream_t)stream);
         return finish(e, "t5a_bwd_dense (no query rows)");
     }
+    p.fp32_math = a->fp32_math;
     p.delta = reinterpret_cast<float*>(a->workspace);
     p.lse2 = p.delta + (int64_t)a->B * a->H * a->M;
     return finish(launch_bwd_dense(p, a->dtype, a->D, a->causal != 0, (hipStream_t)stream), "t5a_bwd_dense");
@@ -414,6 +415,7 @@ int t5a_bwd_varlen(const t5a_varlen_bwd_args* a, t5a_stream_t stream) {
     if (p.n_buckets > 4 * kMaxThresholds) return fail(T5A_ERR_BUCKETS, "num_buckets=%d too large for the backward", p.n_buckets);
     p.dtable = a->bias.table != nullptr ? a->dtable : nullptr;
     if (p.M == 0 || p.N == 0) return fail(T5A_ERR_SHAPE, "max_seqlen_q and max_seqlen_k must be positive");
+    p.fp32_math = a->fp32_math;
     p.delta = reinterpret_cast<float*>(a->workspace);
     p.lse2 = p.delta + (int64_t)a->total_q * a->H;
     return finish(launch_bwd_dense(p, a->dtype, a->D, a->causal != 0, (hipStream_t)stream), "t5a_bwd_varlen");

@@ -139,6 +139,7 @@ struct BwdParams {
     // the statistics (total_q, H)
     const int32_t* cu_q; const int32_t* cu_k; const int32_t* len_q; const int32_t* len_k; int total_q;
     float c1;                         // base-2 score factor: sm_scale * log2(e), or 1 for pre-scaled query rows
+    int fp32_math;                    // nonzero: fp32 matrix cores also for 16-bit inputs at head_dim 64
     int n_buckets;
     const void* table; int table_dtype; int64_t t_sbucket, t_shead;
     BucketSpec bs;

@@ -34,6 +34,11 @@ LOG2E = 1.4426950408889634
 # depend on it; tests pin every path of the run logic with it.
 RUN_LEN = 0
 
+# Backward of 16-bit tensors at head_dim 64.  False: the 16-bit matrix cores, probabilities and dS rounded to the
+# tensors' type before the products that form dq, dk and dv, as the reference's kernels round them
+# (fused_bias_attention.py:575-590).  True: every product on the fp32 matrix cores (about five times slower).
+BACKWARD_FP32_MATH = False
+
 
 def _exact(flag) -> int:
     if isinstance(flag, str):
@@ -247,6 +252,7 @@ def _dense_backward(q, k, v, bias, o, lse, dout, causal, sm_scale, NUM_BUCKETS, 
     a.dtype, a.B, a.H, a.M, a.N, a.D = _dtype_code(q), B, H, M, N, D
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
     a.exact_scores = _exact(exact_scores)
+    a.fp32_math = int(bool(BACKWARD_FP32_MATH))
     b = L.T5ABias()
     keep = None
     if bias is not None:
@@ -445,6 +451,7 @@ def _varlen_backward(q, k, v, bias, o, lse, dout, cu_seqlens_q, cu_seqlens_k, ma
     a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
     a.causal, a.sm_scale = int(bool(causal)), float(sm_scale)
     a.exact_scores = _exact(exact_scores)
+    a.fp32_math = int(bool(BACKWARD_FP32_MATH))
     b = L.T5ABias()
     table = None
     if bias is not None:
