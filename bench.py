@@ -23,7 +23,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                         difference between what the timed launches wrote and that CPU path on row subsets
 
 --leg NAME runs one kernel K times and nothing else, for profiling:
-    dense:BxL[c][:exact|:prescaled]  bwd:BxL[c]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
+    dense:BxL[c][:exact|:prescaled]  bwd:BxL[c][:fp32]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
 --leg NAME --timeline does the same with the measurement build of the library (`python -m turbot5_amd.build --trace`)
 and prints where the work items of the last launch spent their shader-clock cycles.
 """
@@ -223,15 +223,37 @@ def extra_workloads(torch, dev, steps, samples):
         del q, k, v, qs
     out["score_modes"] = modes
 
-    # ---- backward of the dense forward at the headline shape (dq, dk, dv, table gradient; fp32 matrix cores)
-    q, k, v, table = make_inputs(torch, dev, B, H, L, D)
-    o, lse = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0, return_lse=True)
-    gout = torch.randn_like(o)
-    f = lambda: ops._dense_backward(q, k, v, table, o, lse, gout, False, 1.0, 32, 128, None)  # noqa: E731
-    _, ms = time_kernel(torch, f, reps, warm)
-    tf = 10.0 * B * H * D * L * L / (ms * 1e-3) / 1e12
-    out["backward_B16_H12_L1024"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_fp32_mfma_peak": round(tf / PEAK_F32_TFLOPS, 4),
-                                     "note": "three kernels; 2.5 x the forward's FLOPs, fp32 arithmetic whatever the tensors' type"}
+    # ---- backward of the dense forward (dq, dk, dv, table gradient): the headline shape and one sweep point on the
+    # 16-bit matrix cores, the headline shape on the fp32 ones as well (fp32_math), with the largest difference
+    # between the two paths' gradients relative to the gradient's scale
+    bw = {}
+    for bsz, ln in ((B, L), (4, 4096)):
+        q, k, v, table = make_inputs(torch, dev, bsz, H, ln, D, seed=ln if (bsz, ln) != (B, L) else 0)
+        o, lse = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=False, sm_scale=1.0, return_lse=True)
+        gout = torch.randn_like(o)
+        f = lambda: ops._dense_backward(q, k, v, table, o, lse, gout, False, 1.0, 32, 128, None)  # noqa: E731
+        _, ms = time_kernel(torch, f, reps, warm)
+        grads = f()
+        tf = 10.0 * bsz * H * D * ln * ln / (ms * 1e-3) / 1e12
+        bw[f"B{bsz}_L{ln}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+        if (bsz, ln) == (B, L):
+            ops.BACKWARD_FP32_MATH = True
+            try:
+                _, ms32 = time_kernel(torch, f, max(reps // 4, 3), 2, ramp_ms=30.0)
+                ref = f()
+            finally:
+                ops.BACKWARD_FP32_MATH = False
+            tf32 = 10.0 * bsz * H * D * ln * ln / (ms32 * 1e-3) / 1e12
+            bw[f"B{bsz}_L{ln}_fp32_math"] = {"ms": round(ms32, 4), "tflops": round(tf32, 1), "frac_fp32_mfma_peak": round(tf32 / PEAK_F32_TFLOPS, 4)}
+            diff = 0.0
+            for got, want in zip(grads, ref):
+                if got is not None:
+                    diff = max(diff, ((got.float() - want.float()).abs().max() / want.float().abs().max().clamp_min(1e-6)).item())
+            bw["max_rel_diff_16bit_vs_fp32_math"] = round(diff, 5)
+        del q, k, v, o, gout, grads
+    bw["note"] = "three kernels (row statistics, dq pass, dk / dv pass); 2.5 x the forward's FLOPs"
+    out["backward"] = bw
+    q = k = v = o = gout = None
     del q, k, v, o, gout
 
     # ---- head_dim 128 (the T5-3B / 11B head shape): B4 H6 L4096, same FLOPs as the B4 H12 D64 sweep point
@@ -537,7 +559,9 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
         fl = 4.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
     elif name.startswith("bwd:"):
         # the backward kernels alone (dq pass, dk / dv pass, row statistics) on saved forward results: 2.5 x the
-        # forward's FLOPs (five products instead of two), all on the fp32 matrix cores
+        # forward's FLOPs (five products instead of two); bwd:BxL[c]:fp32 runs them on the fp32 matrix cores
+        fp32_math = name.endswith(":fp32")
+        ops.BACKWARD_FP32_MATH = fp32_math
         shape = name.split(":")[1]
         causal = shape.endswith("c")
         b, l = (int(x) for x in shape.rstrip("c").split("x"))
@@ -546,7 +570,7 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
         g = torch.randn_like(o)
         f = lambda: ops._dense_backward(q, k, v, table, o, lse, g, causal, 1.0, 32, 128, None)  # noqa: E731
         fl = 10.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
-        peak = PEAK_F32_TFLOPS
+        peak = PEAK_F32_TFLOPS if fp32_math else PEAK_BF16_TFLOPS
     elif name == "dense_f32_c1":
         # the attention of baseline configuration 1 (T5-small encoder): B4 H8 L512 D64 in fp32, on the fp32 matrix cores
         g = torch.Generator().manual_seed(3)
@@ -640,7 +664,7 @@ def main():
     ap.add_argument("--no-models", action="store_true", help="skip the T5-base model legs (encoder, 100k pass, decoding)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and its checks")
     ap.add_argument("--leg", default=None, metavar="NAME",
-                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], bwd:BxL[c], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
+                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], bwd:BxL[c][:fp32], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
     ap.add_argument("--timeline", action="store_true",
                     help="with --leg: use the measurement build (libt5attn_trace.so) and print the work items' cycle stamps")
     ap.add_argument("--full", action="store_true", help="accepted for compatibility: the default run is the full one")

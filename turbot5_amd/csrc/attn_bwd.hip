@@ -357,8 +357,12 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
     __shared__ float hist_rel[KV ? 1 : 2 * kMaxSaturation + 1];   // dS summed per clamped distance (tiles around the diagonal)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, hh = lane >> 5;
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int own_base = blockIdx.x * kBwdOwn;
+    // Grid: (own blocks, heads, batch).  With a causal mask the own blocks differ in length (a query block sees the
+    // keys up to its own end, a key block the queries from its own start on), and whatever is dispatched last should
+    // be short: the launch is then (heads, batch, own blocks), the slowest index walking the blocks longest first.
+    const int h = CAUSAL ? blockIdx.x : blockIdx.y, b = CAUSAL ? blockIdx.y : blockIdx.z;
+    const int own_block = !CAUSAL ? blockIdx.x : (KV ? blockIdx.z : gridDim.z - 1 - blockIdx.z);
+    const int own_base = own_block * kBwdOwn;
     const int own_row = own_base + wave * 32 + lr;
     int M = p.M, N = p.N;
     int64_t q_first = 0, k_first = 0;
@@ -499,8 +503,14 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
         f32x16 s[NT], dp[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
+            // (dP starts at -delta: the matrix core subtracts it for free)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { s[nt][r] = 0.f; dp[nt][r] = 0.f; }
+            for (int r4 = 0; r4 < 4; ++r4) {
+                f32x4 d4 = {delta_own, delta_own, delta_own, delta_own};
+                if constexpr (KV) d4 = *reinterpret_cast<const f32x4*>(rowstat + kBwdOther + 32 * nt + 8 * r4 + 4 * hh);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { s[nt][4 * r4 + e] = 0.f; dp[nt][4 * r4 + e] = -d4[e]; }
+            }
 #pragma unroll
             for (int k2 = 0; k2 < KS; ++k2) {
                 s[nt] = H16::mfma(*reinterpret_cast<const v8*>(ta + row_off[nt][k2]), fa[k2], s[nt]);
@@ -545,11 +555,11 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
                     for (int half = 0; half < 2; ++half) {
                         const int r4 = 2 * u + half;
                         const int ol0 = 32 * nt + 8 * r4 + 4 * hh;     // first of four consecutive rows of the other kind
-                        f32x4 l4 = {lse2_own, lse2_own, lse2_own, lse2_own}, d4 = {delta_own, delta_own, delta_own, delta_own};
-                        if constexpr (KV) {
-                            l4 = *reinterpret_cast<const f32x4*>(rowstat + ol0);
-                            d4 = *reinterpret_cast<const f32x4*>(rowstat + kBwdOther + ol0);
-                        }
+                        f32x4 l4 = {lse2_own, lse2_own, lse2_own, lse2_own};
+                        if constexpr (KV) l4 = *reinterpret_cast<const f32x4*>(rowstat + ol0);
+                        f32x4 bl4;   // constant bias minus log-sum-exp
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) bl4[e] = bias_c - l4[e];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const int r = 4 * r4 + e, ol = ol0 + e;
@@ -561,12 +571,13 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
                                 x = min(max(rel, -sat), sat) + sat;
                                 bias2 = lut_bias[x];
                             }
-                            float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(c1, s[nt][r], bias2) - l4[e]);
+                            float pv = LUT ? __builtin_amdgcn_exp2f(__builtin_fmaf(c1, s[nt][r], bias2) - l4[e])
+                                           : __builtin_amdgcn_exp2f(__builtin_fmaf(c1, s[nt][r], bl4[e]));
                             if constexpr (CHECK) {
                                 const bool valid = i < M && j < N && (!CAUSAL || rel <= 0);
                                 pv = valid ? pv : 0.f;
                             }
-                            const float ds = pv * (dp[nt][r] - d4[e]);
+                            const float ds = pv * dp[nt][r];
                             pv8[4 * half + e] = pv;
                             ds8[4 * half + e] = ds;
                             if constexpr (!KV) {
@@ -664,8 +675,9 @@ hipError_t launch_bwd_d(const BwdParams& p, bool causal, hipStream_t stream) {
     if constexpr (sizeof(T) == 2 && D == 64) {
         if (p.fp32_math == 0) {
             if (causal) {
-                hipLaunchKernelGGL((bwd16_kernel<T, true, false>), gq, dim3(kBwdThreads), 0, stream, p);
-                if (p.N > 0) hipLaunchKernelGGL((bwd16_kernel<T, true, true>), gk, dim3(kBwdThreads), 0, stream, p);
+                const dim3 cq(p.H, p.B, gq.x), ck(p.H, p.B, gk.x);
+                hipLaunchKernelGGL((bwd16_kernel<T, true, false>), cq, dim3(kBwdThreads), 0, stream, p);
+                if (p.N > 0) hipLaunchKernelGGL((bwd16_kernel<T, true, true>), ck, dim3(kBwdThreads), 0, stream, p);
             } else {
                 hipLaunchKernelGGL((bwd16_kernel<T, false, false>), gq, dim3(kBwdThreads), 0, stream, p);
                 if (p.N > 0) hipLaunchKernelGGL((bwd16_kernel<T, false, true>), gk, dim3(kBwdThreads), 0, stream, p);
