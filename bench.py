@@ -23,7 +23,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                         difference between what the timed launches wrote and that CPU path on row subsets
 
 --leg NAME runs one kernel K times and nothing else, for profiling:
-    dense:BxL[c][:exact|:prescaled]  bwd:BxL[c][:fp32]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
+    dense:BxL[c][:exact|:prescaled]  bwd:BxL[c][:fp32|:d128]  dense_f32_c1  local  block  tglobal  splitk  varlen  varlen_causal  copy
 --leg NAME --timeline does the same with the measurement build of the library (`python -m turbot5_amd.build --trace`)
 and prints where the work items of the last launch spent their shader-clock cycles.
 """
@@ -560,16 +560,18 @@ def run_leg(torch, dev, name, steps, warmup, timeline=False):
     elif name.startswith("bwd:"):
         # the backward kernels alone (dq pass, dk / dv pass, row statistics) on saved forward results: 2.5 x the
         # forward's FLOPs (five products instead of two); bwd:BxL[c]:fp32 runs them on the fp32 matrix cores
+        # (bwd:BxL[c]:d128 is the T5-3B / 11B head shape: 6 heads of 128, the same FLOPs)
         fp32_math = name.endswith(":fp32")
         ops.BACKWARD_FP32_MATH = fp32_math
+        hb, db = (H // 2, 2 * D) if name.endswith(":d128") else (H, D)
         shape = name.split(":")[1]
         causal = shape.endswith("c")
         b, l = (int(x) for x in shape.rstrip("c").split("x"))
-        q, k, v, table = make_inputs(torch, dev, b, H, l, D, seed=l if (b, l) != (B, L) else 0)
+        q, k, v, table = make_inputs(torch, dev, b, hb, l, db, seed=l if (b, l) != (B, L) else 0)
         o, lse = ops.flash_attention_with_fusing_bias(q, k, v, table, causal=causal, sm_scale=1.0, return_lse=True)
         g = torch.randn_like(o)
         f = lambda: ops._dense_backward(q, k, v, table, o, lse, g, causal, 1.0, 32, 128, None)  # noqa: E731
-        fl = 10.0 * b * H * D * (l * (l + 1) // 2 if causal else l * l)
+        fl = 10.0 * b * hb * db * (l * (l + 1) // 2 if causal else l * l)
         peak = PEAK_F32_TFLOPS if fp32_math else PEAK_BF16_TFLOPS
     elif name == "dense_f32_c1":
         # the attention of baseline configuration 1 (T5-small encoder): B4 H8 L512 D64 in fp32, on the fp32 matrix cores
@@ -664,7 +666,7 @@ def main():
     ap.add_argument("--no-models", action="store_true", help="skip the T5-base model legs (encoder, 100k pass, decoding)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg and its checks")
     ap.add_argument("--leg", default=None, metavar="NAME",
-                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], bwd:BxL[c][:fp32], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
+                    help="run only one kernel: dense:BxL[c][:exact|:prescaled], bwd:BxL[c][:fp32|:d128], dense_f32_c1, local, block, tglobal, splitk, varlen, varlen_causal, copy")
     ap.add_argument("--timeline", action="store_true",
                     help="with --leg: use the measurement build (libt5attn_trace.so) and print the work items' cycle stamps")
     ap.add_argument("--full", action="store_true", help="accepted for compatibility: the default run is the full one")

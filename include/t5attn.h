@@ -147,10 +147,11 @@ int t5a_fwd_dense(const t5a_dense_args* args, t5a_stream_t stream);
  * q, k, v, causal, sm_scale, exact_scores and bias as in the forward call; o and lse are what it returned
  * (lse is required); dout is the gradient of o.  dq (B,H,M,D), dk and dv (B,H,N,D) in the tensors' type, any
  * strides {batch, head, row}; dtable (required when bias.table is set): (num_buckets, H) contiguous fp32, overwritten.
- * head_dim 16, 32 or 64.  The table gradient is summed with floating-point atomics: its last bits depend on the
+ * head_dim 16, 32 or 64; 16-bit tensors also 128.  The table gradient is summed with floating-point atomics: its last bits depend on the
  * order of the workgroups.
  * Arithmetic of the backward.  fp32 tensors, head_dim 16 and 32, and any call with fp32_math != 0: every product on
- * the fp32 matrix cores, inputs widened on their way in.  16-bit tensors at head_dim 64 with fp32_math == 0: the
+ * the fp32 matrix cores, inputs widened on their way in (head_dim up to 64).  16-bit tensors at head_dim 64 and 128
+ * with fp32_math == 0: the
  * 16-bit matrix cores -- the score and dP products take the inputs as they are, and the probabilities and dS are
  * rounded to the tensors' type before the products that form dq, dk and dv, as the reference rounds them
  * (fused_bias_attention.py:575-590); sums, the softmax statistics and the table gradient stay in fp32.  About

@@ -98,6 +98,32 @@ def test_16_bit_gradients_over_long_rows(gpu_device, dtype, causal, M, N):
         check(name, g, w, TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,H,M,N", [(2, 2, 256, 256), (1, 2, 200, 333), (1, 2, 700, 1100), (1, 1, 1, 300), (1, 2, 130, 70)])
+def test_16_bit_gradients_at_head_dim_128(gpu_device, dtype, causal, B, H, M, N):
+    """The T5-3B / 11B head shape: three passes (dq, dk, dv) over rows of 256 bytes.  fp32 tensors and fp32_math have
+    no backward at this head_dim and say so."""
+    from turbot5_amd import ops
+    D = 128
+    q, k, v = rnd(B, H, M, D, seed=81, dtype=dtype), rnd(B, H, N, D, seed=82, dtype=dtype), rnd(B, H, N, D, seed=83, dtype=dtype)
+    table = rnd(32, H, seed=84, scale=1.0)
+    dout = rnd(B, H, M, D, seed=85, scale=1.0, dtype=dtype)
+    _, wq, wk, wv, wt = oracle_grads(q, k, v, table, dout, causal, None)
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    ops.flash_attention_with_fusing_bias(dq, dk, dv, dt, causal=causal).backward(dout.to(gpu_device))
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv), ("dtable", dt.grad, wt)):
+        check(name, g, w, TOL[dtype])
+
+
+def test_head_dim_128_backward_refuses_fp32(gpu_device):
+    from turbot5_amd import ops
+    q, k, v = (rnd(1, 1, 64, 128, seed=86 + i).to(gpu_device).requires_grad_(True) for i in range(3))
+    out = ops.flash_attention_with_fusing_bias(q, k, v, None)
+    with pytest.raises(NotImplementedError, match="head_dim 128"):
+        out.sum().backward()
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_16_bit_gradients_on_the_fp32_matrix_cores_and_of_strided_views(gpu_device, monkeypatch, causal):
     """fp32_math: the fp32 kernels also for 16-bit tensors at head_dim 64 (they only round their results), so the two

@@ -298,7 +298,8 @@ int t5a_bwd_dense(const t5a_dense_bwd_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
     if (rc) return rc;
-    if (a->D == 128) return fail(T5A_ERR_HEAD_DIM, "the backward kernels hold a row's head_dim in registers: head_dim 16, 32 or 64");
+    if (a->D == 128 && (a->dtype == T5A_F32 || a->fp32_math != 0))
+        return fail(T5A_ERR_HEAD_DIM, "backward at head_dim 128: 16-bit tensors on the 16-bit matrix cores only (the fp32 kernels hold a row's head_dim in registers: 16, 32 or 64)");
     const int unit = a->dtype == T5A_F32 ? 4 : 8;
     if (a->B < 0 || a->H <= 0 || a->M < 0 || a->N < 0) return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d M=%d N=%d", a->B, a->H, a->M, a->N);
     if (a->B == 0) return T5A_OK;
@@ -370,7 +371,8 @@ int t5a_bwd_varlen(const t5a_varlen_bwd_args* a, t5a_stream_t stream) {
     if (a == nullptr) return fail(T5A_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->D);
     if (rc) return rc;
-    if (a->D == 128) return fail(T5A_ERR_HEAD_DIM, "the backward kernels hold a row's head_dim in registers: head_dim 16, 32 or 64");
+    if (a->D == 128 && (a->dtype == T5A_F32 || a->fp32_math != 0))
+        return fail(T5A_ERR_HEAD_DIM, "backward at head_dim 128: 16-bit tensors on the 16-bit matrix cores only (the fp32 kernels hold a row's head_dim in registers: 16, 32 or 64)");
     const int unit = a->dtype == T5A_F32 ? 4 : 8;
     if (a->B < 0 || a->H <= 0 || a->total_q < 0 || a->total_k < 0 || a->max_seqlen_q < 0 || a->max_seqlen_k < 0)
         return fail(T5A_ERR_SHAPE, "bad sizes B=%d H=%d total_q=%d total_k=%d", a->B, a->H, a->total_q, a->total_k);

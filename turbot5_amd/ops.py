@@ -232,8 +232,8 @@ def _dense_backward(q, k, v, bias, o, lse, dout, causal, sm_scale, NUM_BUCKETS, 
     """-> dq, dk, dv, dbias (fp32 (NUM_BUCKETS, H), or None without a table); t5a_bwd_dense"""
     B, H, M, D = q.shape
     N = k.shape[2]
-    if D == 128:
-        raise NotImplementedError("the backward kernels cover head_dim 16, 32 and 64")
+    if D == 128 and (q.dtype == torch.float32 or BACKWARD_FP32_MATH):
+        raise NotImplementedError("backward at head_dim 128: bf16 / fp16 tensors only (the fp32 kernels cover head_dim 16, 32 and 64)")
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
     q_, k_, v_, o_, g_ = (_kernel_ready(t) for t in (q, k, v, o, dout))
@@ -301,7 +301,7 @@ def flash_attention_with_fusing_bias(q, k, v, bias, causal=False, sm_scale=None,
     (NUM_BUCKETS, H) table or None.  ``causal`` selects the causal mask and the
     unidirectional buckets together.  ``sm_scale=None`` means 1/sqrt(D).  Returns
     a tensor shaped and strided like q (``empty_like``), plus the (B,H,M) fp32
-    log-sum-exp when ``return_lse``.  Differentiable in q, k, v and the table (head_dim up to 64), as the
+    log-sum-exp when ``return_lse``.  Differentiable in q, k, v and the table (fp32 tensors: head_dim up to 64), as the
     reference's autograd function is (fused_bias_attention.py:821-873).
     """
     needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (q, k, v, bias))
@@ -419,8 +419,8 @@ def _varlen_backward(q, k, v, bias, o, lse, dout, cu_seqlens_q, cu_seqlens_k, ma
                      NUM_BUCKETS, MAX_DISTANCE, seq_lens_q, seq_lens_k, exact_scores):
     """-> dq, dk, dv, dbias (fp32 (NUM_BUCKETS, H) or None); t5a_bwd_varlen"""
     total_q, H, D = q.shape
-    if D == 128:
-        raise NotImplementedError("the backward kernels cover head_dim 16, 32 and 64")
+    if D == 128 and (q.dtype == torch.float32 or BACKWARD_FP32_MATH):
+        raise NotImplementedError("backward at head_dim 128: bf16 / fp16 tensors only (the fp32 kernels cover head_dim 16, 32 and 64)")
     B = cu_seqlens_q.numel() - 1
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
