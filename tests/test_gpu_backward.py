@@ -271,6 +271,33 @@ def test_packed_gradients_match_autograd_through_the_oracle(gpu_device, dtype, c
         check(name, g, w, tol)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_packed_gradients_at_head_dim_128(gpu_device, causal):
+    """The packed backward through the head_dim-128 passes (bf16), sequence by sequence against the oracle."""
+    from turbot5_amd import ops
+    H, D = 2, 128
+    lens = [150, 1, 260, 64]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    total = int(cu[-1])
+    q, k, v = (rnd(total, H, D, seed=90 + i, dtype=torch.bfloat16) for i in range(3))
+    table = rnd(32, H, seed=93, scale=1.0)
+    dout = rnd(total, H, D, seed=94, scale=1.0, dtype=torch.bfloat16)
+    wq, wk, wv = (torch.zeros(total, H, D) for _ in range(3))
+    wt = torch.zeros(32, H)
+    for b, n in enumerate(lens):
+        s, e = int(cu[b]), int(cu[b + 1])
+        _, gq, gk, gv, gt = oracle_grads(*(t[s:e].transpose(0, 1)[None] for t in (q, k, v)), table,
+                                         dout[s:e].transpose(0, 1)[None], causal, 1.0)
+        wq[s:e], wk[s:e], wv[s:e] = (g[0].transpose(0, 1) for g in (gq, gk, gv))
+        wt += gt
+    dq, dk, dv, dt = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v, table))
+    dcu = cu.to(gpu_device)
+    out = ops.flash_attention_with_fusing_bias_varlen(dq, dk, dv, dt, dcu, dcu, max(lens), max(lens), causal=causal, sm_scale=1.0)
+    out.backward(dout.to(gpu_device))
+    for name, g, w in (("dq", dq.grad, wq), ("dk", dk.grad, wk), ("dv", dv.grad, wv), ("dtable", dt.grad, wt)):
+        check(name, g, w, 2e-2)
+
+
 def test_packed_gradients_of_a_padded_batch_in_place(gpu_device):
     """A right-padded (B, L) batch run in place (cu = multiples of L, seq_lens = the lengths), keys longer than the
     queries in one call (cached decoding shape): padding rows get zero gradients, the rest matches the oracle."""
