@@ -147,6 +147,54 @@ def test_16_bit_gradients_on_the_fp32_matrix_cores_and_of_strided_views(gpu_devi
                 check(f"dtable fp32_math={fp32_math}", dt.grad, wt, tol)
 
 
+def test_the_two_arithmetic_paths_agree_on_random_shapes(gpu_device, monkeypatch):
+    """Seeded random shapes (M and N from 1 to 1500, either larger, causal or not, with and without a table, packed
+    batches with random lengths): the 16-bit kernels against the fp32 kernels on the same inputs, which the other
+    tests pin to the oracle.  Size-independent, so it also runs shapes too large for autograd on the CPU."""
+    import random
+    from turbot5_amd import ops
+    rng = random.Random(7)
+
+    def both(fn):
+        res = []
+        for fp32_math in (False, True):
+            monkeypatch.setattr(ops, "BACKWARD_FP32_MATH", fp32_math)
+            res.append(fn())
+        return res
+
+    for case in range(14):
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        causal, with_table = rng.random() < 0.5, rng.random() < 0.7
+        H = rng.choice([1, 2, 3])
+        if case % 3 == 2:     # packed
+            lens = [rng.randint(1, 700) for _ in range(rng.randint(1, 5))]
+            cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=gpu_device)
+            total = sum(lens)
+            q, k, v, dout = (rnd(total, H, 64, seed=100 * case + i, dtype=dtype).to(gpu_device) for i in range(4))
+            shape = f"packed {lens}"
+        else:
+            B, M, N = rng.choice([1, 2]), rng.randint(1, 1500), rng.randint(1, 1500)
+            q, dout = (rnd(B, H, M, 64, seed=100 * case + i, dtype=dtype).to(gpu_device) for i in range(2))
+            k, v = (rnd(B, H, N, 64, seed=100 * case + 2 + i, dtype=dtype).to(gpu_device) for i in range(2))
+            shape = f"B{B} M{M} N{N}"
+        table = rnd(32, H, seed=100 * case + 9, scale=1.0).to(gpu_device) if with_table else None
+
+        def grads():
+            leaves = [t.clone().requires_grad_(True) for t in (q, k, v)] + ([table.clone().requires_grad_(True)] if with_table else [])
+            tab = leaves[3] if with_table else None
+            if case % 3 == 2:
+                out = ops.flash_attention_with_fusing_bias_varlen(*leaves[:3], tab, cu, cu, max(lens), max(lens), causal=causal, sm_scale=1.0)
+            else:
+                out = ops.flash_attention_with_fusing_bias(*leaves[:3], tab, causal=causal, sm_scale=1.0)
+            out.backward(dout)
+            return [t.grad for t in leaves]
+
+        fast, exact = both(grads)
+        for name, g, w in zip(("dq", "dk", "dv", "dtable"), fast, exact):
+            assert torch.isfinite(g).all(), (case, shape, name)
+            check(f"case {case} {shape} causal={causal} {dtype} {name}", g, w.float().cpu(), 2e-2)
+
+
 def test_gradients_with_prescaled_query_rows(gpu_device):
     """exact_scores="prescaled": the rows carry log2(e), the score factor of the op is ln 2 -- and so is the
     factor on dq and dk.  Differentiated through ops.prescaled_query down to the hidden states and the weight."""
