@@ -1707,7 +1707,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
             for (int j = 0; j < 8; ++j) pe[j] = exp_pair(st[0][2 * j], st[0][2 * j + 1], (j & 1) ? lt1 : lt0);
         }
     };
-    auto dense_halves = [&](int vstage, const v8 (&ka)[NT][KS], f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+    // (LAST: the step that reaches the item's last tile -- no S products and no early exponentials for a tile behind it)
+    auto dense_halves = [&](auto last_c, int vstage, const v8 (&ka)[NT][KS], f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        constexpr bool LAST = decltype(last_c)::value;
         if constexpr (V2) {
             static_assert(!V2 || (NT == 2 && KS == 4 && DT == 2), "four groups of 16 keys, two products each");
             typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -1726,11 +1728,13 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 pl[i] = exp_pair(st[1][2 * i], st[1][2 * i + 1], (i & 1) ? lt1 : lt0);
-                if (i >= 2) st_next[i & 1] = E::mfma(ka[i & 1][i >> 1], qf[i >> 1], st_next[i & 1]);
+                if constexpr (!LAST) {
+                    if (i >= 2) st_next[i & 1] = E::mfma(ka[i & 1][i >> 1], qf[i >> 1], st_next[i & 1]);
+                }
                 if (i >= 4) vread((i - 4) >> 1, (i - 4) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (exact) {
+            if constexpr (exact && !LAST) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -1752,7 +1756,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) { st[nt][r] -= delta; st_next[nt][r] -= delta; }
+                    for (int r = 0; r < 16; ++r) { st[nt][r] -= delta; if constexpr (!LAST) st_next[nt][r] -= delta; }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -1778,7 +1782,8 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                                        : u32x4{pl[4 * g - 8], pl[4 * g - 7], pl[4 * g - 6], pl[4 * g - 5]};
                 ot[dt] = E::mfma(vf[g][dt], __builtin_bit_cast(v8, pw), ot[dt]);
                 if (i < 4) vread(2 + (i >> 1), i & 1);
-                pn[i] = exp_pair(st_next[0][2 * i], st_next[0][2 * i + 1], (i & 1) ? lt1 : lt0);
+                if constexpr (!LAST) pn[i] = exp_pair(st_next[0][2 * i], st_next[0][2 * i + 1], (i & 1) ? lt1 : lt0);
+                else pn[i] = 0u;
                 __builtin_amdgcn_sched_barrier(0);
             }
             // (pinned here: the compiler otherwise sinks the last step's exponentials of an unrolled group of four
@@ -1793,12 +1798,24 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     // compile time.
     int fc_until = 0, fc_side = 0;   // dense fast steps: class of the next tile, valid for tiles below fc_until
     bool fc_lut = false;
-    auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+    auto fast_step_impl = [&](int t, auto st_c, auto last_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
         constexpr int ST = decltype(st_c)::value;
+        constexpr bool LAST = decltype(last_c)::value;   // nothing follows tile t: no product for a tile t + 1
         if constexpr (DENSE) cursor_dma(ST, (ST + 3) & 3);
         else if constexpr (CURSOR) { dma_next(false, ST); dma_next(true, (ST + 3) & 3); }
         else { dma_tile(t + 4, false, ST); dma_tile(t + 3, true, (ST + 3) & 3); }
         v8 ka[NT][KS];
+        if constexpr (LAST) {
+            static_assert(!LAST || V2, "only the dense steps without row maxima have this form");
+            head_refill = false;
+            dense_halves(last_c, ST, ka, st, st_next);
+            tc.skip = true;
+            T5A_PHASE(0);
+            step_wait();
+            barrier_lds_only();
+            T5A_PHASE(1);
+            return;
+        }
         read_k((ST + 1) & 3, ka);
         TileClass nx;
         if constexpr (win_lut) {   // one segment, every tile takes its accumulator input from the LUT: nothing to look up
@@ -1829,7 +1846,7 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 st_next[0] = E::mfma(ka[0][0], qf[0], cm);   // cm stays live: untied accumulator input
                 st_next[1] = E::mfma(ka[1][0], qf[0], cm);
             }
-            if constexpr (V2) dense_halves(ST, ka, st, st_next);
+            if constexpr (V2) dense_halves(last_c, ST, ka, st, st_next);
             else fused_halves(live, ST, ka, st, st_next);
         } else {
             __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): one wait for all K fragments instead of one per MFMA
@@ -1843,6 +1860,9 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         step_wait();
         barrier_lds_only();
         T5A_PHASE(1);
+    };
+    auto fast_step = [&](int t, auto st_c, f32x16 (&st)[NT], f32x16 (&st_next)[NT]) {
+        fast_step_impl(t, st_c, std::false_type{}, st, st_next);
     };
     // number of consecutive tiles from t on that are neither skipped nor masked
     auto plain_run = [&](int t) {
@@ -1959,12 +1979,18 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                 // stage holds zeros or a tile of the next q tile) and nobody consumes it, so the run may end
                 // exactly there.
                 const int run = plain_run(t);
-                const int fast = t + run >= ntiles ? run : run - 1;   // steps from here on that can be fast ones
+                const bool ends = t + run >= ntiles;                   // the plain tiles reach the item's last tile
+                const int fast = ends ? run : run - 1;                 // steps from here on that can be fast ones
                 int quads = fast >> 2;
+                // (dense kinds) a run that ends with the item's last tile on a group of four: that group is a copy of
+                // its own behind the loop, whose last step leaves the product for a tile behind it out
+                // (not with exact scores: that instantiation has no registers left for the copy)
+                const bool peel = V2 && !exact && ends && quads > 0 && (fast & 3) == 0;
+                if (peel) --quads;
                 // dense kinds: two more fast steps behind the groups of four (ring stages 0 and 1), so that the tail of
                 // a short or causal item takes fewer general steps
                 const bool pair = V2 && fast >= 2 && (fast & 3) >= 2;
-                const bool ran_fast = quads > 0 || pair;
+                const bool ran_fast = quads > 0 || pair || peel;
                 if (ran_fast) {
                     tc = classify(t);
                     if constexpr (DENSE) { cursor_seek(t + 4, t + 3); fc_until = 0; }
@@ -1977,6 +2003,15 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
                     fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
                     fast_step(t + 3, std::integral_constant<int, 3>{}, stb, sta);
                     --quads; t += 4;
+                }
+                if constexpr (V2 && !exact) {
+                    if (peel) {
+                        fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
+                        fast_step(t + 1, std::integral_constant<int, 1>{}, stb, sta);
+                        fast_step(t + 2, std::integral_constant<int, 2>{}, sta, stb);
+                        fast_step_impl(t + 3, std::integral_constant<int, 3>{}, std::true_type{}, stb, sta);
+                        t += 4;
+                    }
                 }
                 if (pair) {
                     fast_step(t, std::integral_constant<int, 0>{}, sta, stb);
