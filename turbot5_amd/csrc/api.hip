@@ -312,6 +312,9 @@ int t5a_bwd_dense(const t5a_dense_bwd_args* a, t5a_stream_t stream) {
         if ((rc = check_tensor(t.name, t.ptr, t.st, 3, unit))) return rc;
     }
     if (a->M > 0 && a->lse == nullptr) return fail(T5A_ERR_NULL, "lse is NULL");
+    // (the kernels address the rows of a (batch, head) slice with 32-bit byte offsets)
+    for (auto& t : ts)
+        if (t.rows > 0 && (rc = check_rows(t.name, t.rows, t.st[2], a->dtype))) return rc;
     const int64_t need = t5a_bwd_workspace_bytes(a->B, a->H, a->M);
     if (a->M > 0 && (a->workspace == nullptr || a->workspace_bytes < need))
         return fail(T5A_ERR_WORKSPACE, "t5a_bwd_dense: workspace of %lld bytes needed, %lld given", (long long)need, (long long)a->workspace_bytes);
@@ -383,8 +386,11 @@ int t5a_bwd_varlen(const t5a_varlen_bwd_args* a, t5a_stream_t stream) {
     struct { const char* name; const void* ptr; const int64_t* st; } ts[] = {
         {"q", a->q, a->q_strides}, {"o", a->o, a->o_strides}, {"dout", a->dout, a->dout_strides}, {"dq", a->dq, a->dq_strides},
         {"k", a->k, a->k_strides}, {"v", a->v, a->v_strides}, {"dk", a->dk, a->dk_strides}, {"dv", a->dv, a->dv_strides}};
-    for (auto& t : ts)
+    for (auto& t : ts) {
         if ((rc = check_tensor(t.name, t.ptr, t.st, 2, unit))) return rc;
+        // (a sequence's rows are addressed with 32-bit byte offsets from its first row)
+        if ((rc = check_rows(t.name, a->max_seqlen_q > a->max_seqlen_k ? a->max_seqlen_q : a->max_seqlen_k, t.st[0], a->dtype))) return rc;
+    }
     if (a->lse == nullptr) return fail(T5A_ERR_NULL, "lse is NULL");
     const int64_t need = t5a_bwd_varlen_workspace_bytes(a->total_q, a->H);
     if (a->workspace == nullptr || a->workspace_bytes < need)

@@ -343,6 +343,22 @@ template <> struct Half16<_Float16> {
 // rows x 64 bytes at a time)
 __device__ __forceinline__ int tile_swz(int row) { return ((row >> 1) & 7) ^ (((row >> 1) & 1) << 2); }
 
+// LDS-DMA: a wavefront instruction fetches 64 x 16 bytes at per-lane byte offsets of a buffer (zeros past its end) and
+// writes them to 1 KB of consecutive LDS addresses in lane order, without passing through registers.  Issued from
+// assembly, so the wait for it (vmcnt) is the kernel's own.
+__device__ __forceinline__ u32x4 dma_rsrc(const void* base, unsigned bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+    return u32x4{(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+                 (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu)),
+                 (unsigned)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+}
+__device__ __forceinline__ void dma_16(u32x4 rs, unsigned lds_addr, int voffset) {
+    const u32x4 rsrc = {(unsigned)__builtin_amdgcn_readfirstlane((int)rs[0]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[1]),
+                        (unsigned)__builtin_amdgcn_readfirstlane((int)rs[2]), (unsigned)__builtin_amdgcn_readfirstlane((int)rs[3])};
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+
 template <typename T, bool CAUSAL, bool KV>
 __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p) {
     constexpr int D = 64, DT = 2, KS = 4, NT = kBwdOther / 32;
@@ -420,23 +436,36 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
         else t_lo = max(0, own_base - P) / kBwdOther;
     }
 
-    // staging: thread -> two 16-byte chunks of each tile (row = idx / 8, chunk = idx % 8)
+    // staging by LDS-DMA: a tile is 8 slabs of 1 KB (8 rows); wavefront w requests slabs 2 w and 2 w + 1 of each of
+    // the two tiles.  The chunk swizzle is applied on the source side: the lane that writes physical chunk pc of row r
+    // fetches logical chunk pc ^ swizzle(r).  Rows past the end of the tensor are out of the descriptor's range and
+    // arrive as zeros.  (Slices stay below 2 GiB -- checked on the host -- so 32-bit offsets do.)
     const T* src_a = KV ? qp : kp;
     const T* src_b = KV ? gp : vp;
-    const int64_t a_sr = KV ? p.q_sr : p.k_sr, b_sr = KV ? p.do_sr : p.v_sr;
-    u32x4 ra[2], rb[2];
+    const int a_srb = (int)(KV ? p.q_sr : p.k_sr) * 2, b_srb = (int)(KV ? p.do_sr : p.v_sr) * 2;     // row strides in bytes
+    const u32x4 rs_a = dma_rsrc(src_a, n_other > 0 ? (unsigned)(n_other - 1) * (unsigned)a_srb + D * 2 : 0u);
+    const u32x4 rs_b = dma_rsrc(src_b, n_other > 0 ? (unsigned)(n_other - 1) * (unsigned)b_srb + D * 2 : 0u);
+    int dma_a[2], dma_b[2];     // this lane's byte offsets inside a tile, per slab
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int row = (2 * wave + c) * 8 + (lane >> 3), ch = (lane & 7) ^ tile_swz(row);
+        dma_a[c] = row * a_srb + ch * 16;
+        dma_b[c] = row * b_srb + ch * 16;
+    }
+    const unsigned lds_a = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)&ta2[0][0];
+    const unsigned lds_b = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)&tb2[0][0];
     float rstat = 0.f;
-    auto fetch = [&](int t) {
+    auto request = [&](int t, int buf) {     // tile t into buffer buf: four requests per wavefront
         const int o0 = t * kBwdOther;
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            const int idx = tid + c * kBwdThreads, row = idx >> 3, ch = idx & 7;
-            ra[c] = u32x4{0u, 0u, 0u, 0u}; rb[c] = u32x4{0u, 0u, 0u, 0u};
-            if (o0 + row < n_other) {
-                ra[c] = *reinterpret_cast<const u32x4*>(src_a + (int64_t)(o0 + row) * a_sr + 8 * ch);
-                rb[c] = *reinterpret_cast<const u32x4*>(src_b + (int64_t)(o0 + row) * b_sr + 8 * ch);
-            }
+            const unsigned at = (unsigned)buf * (kBwdOther * D * 2) + (2 * wave + c) * 1024u;
+            dma_16(rs_a, lds_a + at, o0 * a_srb + dma_a[c]);
+            dma_16(rs_b, lds_b + at, o0 * b_srb + dma_b[c]);
         }
+    };
+    auto fetch_stat = [&](int t) {
+        const int o0 = t * kBwdOther;
         if (KV && tid < 2 * kBwdOther) {
             const int row = tid & (kBwdOther - 1);
             rstat = tid < kBwdOther ? INFINITY : 0.f;
@@ -444,17 +473,8 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
                 rstat = tid < kBwdOther ? p.lse2[stat_base + (o0 + row) * stat_sr] : p.delta[stat_base + (o0 + row) * stat_sr];
         }
     };
-    auto stage = [&](int buf) {
-        T* ta = ta2[buf]; T* tb = tb2[buf];
-        float* rowstat = rowstat2[buf];
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int idx = tid + c * kBwdThreads, row = idx >> 3, ch = idx & 7;
-            const int at = row * D + ((ch ^ tile_swz(row)) * 8);
-            *reinterpret_cast<u32x4*>(ta + at) = ra[c];
-            *reinterpret_cast<u32x4*>(tb + at) = rb[c];
-        }
-        if (KV && tid < 2 * kBwdOther) rowstat[tid] = rstat;
+    auto stage_stat = [&](int buf) {
+        if (KV && tid < 2 * kBwdOther) rowstat2[buf][tid] = rstat;
     };
     // row reads: element offsets of this lane's chunk (2 s + hh) of row 32 nt + lr
     int row_off[NT][KS];
@@ -491,12 +511,15 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
         for (int r = 0; r < 16; ++r) { acc_a[dt][r] = 0.f; acc_b[dt][r] = 0.f; }
     float sum_lo = 0.f, sum_hi = 0.f;
 
-    if (t_lo < t_hi) { fetch(t_lo); stage(0); }
-    if (t_lo + 1 < t_hi) fetch(t_lo + 1);
-    __syncthreads();     // tile t_lo and the LUT are written
+    // Tile t + 1 is requested when the barrier at the top of tile t has shown that every wavefront is done with the
+    // buffer it goes into, and has all of tile t's work to arrive in.
+    if (t_lo < t_hi) { request(t_lo, 0); fetch_stat(t_lo); stage_stat(0); }
     for (int t = t_lo; t < t_hi; ++t) {
         const int o0 = t * kBwdOther;
         const int buf = (t - t_lo) & 1;
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this wavefront's requests for tile t have landed
+        __syncthreads();                        // ... and everybody's; the other buffer is free (and, first time round, the LUT written)
+        if (t + 1 < t_hi) { request(t + 1, buf ^ 1); fetch_stat(t + 1); }
         const T* ta = ta2[buf]; const T* tb = tb2[buf];
         const float* rowstat = rowstat2[buf];
         (void)rowstat;
@@ -623,10 +646,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
         else if (!use_lut) second_stage(std::true_type{}, std::false_type{});
         else second_stage(std::true_type{}, std::true_type{});
         if (side == 1) sum_lo += tile_sum; else if (side == 2) sum_hi += tile_sum;
-        // the next tile goes into the other buffer, whose readers passed the barrier at the end of the previous round
-        if (t + 1 < t_hi) stage(buf ^ 1);
-        __syncthreads();
-        if (t + 2 < t_hi) fetch(t + 2);
+        if (t + 1 < t_hi) stage_stat(buf ^ 1);
     }
 
     const float scale = p.c1 * 0.6931471805599453f;
