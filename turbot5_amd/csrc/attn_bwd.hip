@@ -63,39 +63,59 @@ template <typename T> __device__ __forceinline__ void store4(T* p, f32x4 x) {
     }
 }
 
+// rows per block of bwd_rows_kernel: up to eight threads share a row, 16 bytes per load, so that a wavefront's loads
+// cover whole rows (one thread per row reads with a stride of a row and takes twice as long)
+template <typename T, int D> struct RowsGeom {
+    static constexpr int CH = D * (int)sizeof(T) / 16;      // 16-byte chunks per row
+    static constexpr int TPR = CH < 8 ? CH : 8;             // threads per row
+    static constexpr int CPT = CH / TPR;                    // chunks per thread
+    static constexpr int ROWS = 256 / TPR;                  // rows per block
+    static constexpr int EPC = 16 / (int)sizeof(T);         // elements per chunk
+};
+
 template <typename T, int D>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const BwdParams p) {
+    using G = RowsGeom<T, D>;
     // dense: row = (b, h, i) flattened, statistics (B,H,M); packed: row = (token, h) flattened, statistics (total_q, H)
-    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int sub = threadIdx.x % G::TPR;
+    const int64_t row = (int64_t)blockIdx.x * G::ROWS + threadIdx.x / G::TPR;
     const bool packed = p.cu_q != nullptr;
     const int64_t rows = packed ? (int64_t)p.total_q * p.H : (int64_t)p.B * p.H * p.M;
     // the table gradient is accumulated with atomics by the dq kernel: clear it here, ahead of that launch
     if (p.dtable != nullptr) {
         const int64_t n = (int64_t)p.n_buckets * p.H;
-        for (int64_t x = row; x < n; x += (int64_t)gridDim.x * 256) p.dtable[x] = 0.f;
+        for (int64_t x = (int64_t)blockIdx.x * 256 + threadIdx.x; x < n; x += (int64_t)gridDim.x * 256) p.dtable[x] = 0.f;
     }
-    if (row >= rows) return;
-    int64_t o_off, g_off;
-    if (packed) {
-        const int64_t tok = row / p.H;
-        const int h = (int)(row - tok * p.H);
-        o_off = tok * p.o_sr + (int64_t)h * p.o_sh;
-        g_off = tok * p.do_sr + (int64_t)h * p.do_sh;
-    } else {
-        const int i = (int)(row % p.M);
-        const int64_t bh = row / p.M;
-        const int h = (int)(bh % p.H), b = (int)(bh / p.H);
-        o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)i * p.o_sr;
-        g_off = (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + (int64_t)i * p.do_sr;
-    }
-    const T* o = reinterpret_cast<const T*>(p.o) + o_off;
-    const T* g = reinterpret_cast<const T*>(p.dout) + g_off;
     float acc = 0.f;
+    if (row < rows) {
+        int64_t o_off, g_off;
+        if (packed) {
+            const int64_t tok = row / p.H;
+            const int h = (int)(row - tok * p.H);
+            o_off = tok * p.o_sr + (int64_t)h * p.o_sh;
+            g_off = tok * p.do_sr + (int64_t)h * p.do_sh;
+        } else {
+            const int i = (int)(row % p.M);
+            const int64_t bh = row / p.M;
+            const int h = (int)(bh % p.H), b = (int)(bh / p.H);
+            o_off = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + (int64_t)i * p.o_sr;
+            g_off = (int64_t)b * p.do_sb + (int64_t)h * p.do_sh + (int64_t)i * p.do_sr;
+        }
+        const T* o = reinterpret_cast<const T*>(p.o) + o_off;
+        const T* g = reinterpret_cast<const T*>(p.dout) + g_off;
 #pragma unroll
-    for (int c = 0; c < D / 4; ++c) {
-        const f32x4 x = load4(o + 4 * c), y = load4(g + 4 * c);
-        acc += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+        for (int c = 0; c < G::CPT; ++c)
+#pragma unroll
+            for (int q4 = 0; q4 < G::EPC / 4; ++q4) {
+                const int at = (sub * G::CPT + c) * G::EPC + 4 * q4;
+                const f32x4 x = load4(o + at), y = load4(g + at);
+                acc += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+            }
     }
+    // (every lane takes part in the exchange; the threads of a row are neighbours in one wavefront)
+#pragma unroll
+    for (int off = 1; off < G::TPR; off <<= 1) acc += __shfl_xor(acc, off, 64);
+    if (row >= rows || sub != 0) return;
     p.delta[row] = acc;
     const float l = p.lse[row];
     // a row without a visible key: +inf makes every exp2(score - lse2) of the row 0
@@ -1017,7 +1037,7 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_d128_kernel(const BwdPar
 template <typename T, int D>
 hipError_t launch_bwd_d(const BwdParams& p, bool causal, hipStream_t stream) {
     const int64_t rows = p.cu_q != nullptr ? (int64_t)p.total_q * p.H : (int64_t)p.B * p.H * p.M;
-    hipLaunchKernelGGL((bwd_rows_kernel<T, D>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((bwd_rows_kernel<T, D>), dim3((unsigned)((rows + RowsGeom<T, D>::ROWS - 1) / RowsGeom<T, D>::ROWS)), dim3(256), 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const dim3 gq((p.M + kBwdOwn - 1) / kBwdOwn, p.H, p.B), gk((p.N + kBwdOwn - 1) / kBwdOwn, p.H, p.B);
@@ -1052,7 +1072,7 @@ hipError_t launch_bwd_d128(const BwdParams& p, bool causal, hipStream_t stream) 
     } else {
         if (p.fp32_math != 0) return hipErrorInvalidValue;     // (the fp32 kernels hold a row's head_dim in registers: up to 64)
         const int64_t rows = p.cu_q != nullptr ? (int64_t)p.total_q * p.H : (int64_t)p.B * p.H * p.M;
-        hipLaunchKernelGGL((bwd_rows_kernel<T, 128>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((bwd_rows_kernel<T, 128>), dim3((unsigned)((rows + RowsGeom<T, 128>::ROWS - 1) / RowsGeom<T, 128>::ROWS)), dim3(256), 0, stream, p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const unsigned nq = (p.M + kBwdOwn - 1) / kBwdOwn, nk = (p.N + kBwdOwn - 1) / kBwdOwn;
