@@ -334,11 +334,6 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
     T* Ks = Vs + NSV * V_TILE;                  // [NSK][K_TILE]
     float* lut = reinterpret_cast<float*>(Ks + NSK * K_TILE);   // [4][4*quads]
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int lr = lane & 31;
-    const int hh = lane >> 5;
 
     // ---------------------------------------------------------------- work item
     // Consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
@@ -403,6 +398,14 @@ __global__ __launch_bounds__(NTHREADS, (D >= 128 && sizeof(T) == 4) ? 1 : kWorkg
         if (BLOCK && p.block_items > 0 && w >= p.block_items) run_left = 1;   // a key split of the global rows: one pass
     }
     for (;;) {
+    // (runs of q tiles: the thread index is made opaque once per pass; otherwise every per-lane constant of the set-up
+    // is computed once before this loop -- ahead of the first tile requests -- and kept, or spilled, across all passes)
+    int tid = threadIdx.x;
+    if constexpr (RUNS) asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 31;
+    const int hh = lane >> 5;
     int b = 0, h = 0, qt = 0, Mseq = 0, Nseq = 0, split = 0, key0 = 0;
     bool gsplit = false;     // block pattern: this item is a key split of the global rows
     int key_lo = 0;          // windowed patterns: first key of the sequence (a batch padded on the left)
