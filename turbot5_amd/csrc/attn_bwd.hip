@@ -421,16 +421,6 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
     const int64_t stat_sr = p.cu_q != nullptr ? p.H : 1;
     const int64_t stat_base = p.cu_q != nullptr ? q_first * p.H + h : ((int64_t)b * p.H + h) * p.M;
 
-    if (has_bias) {
-        for (int x = tid; x <= 2 * sat; x += kBwdThreads) {
-            const int bk = bucket_of(p.bs, x - sat);
-            lut_bias[x] = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * 1.4426950408889634f;
-            if constexpr (!KV) { lut_bucket[x] = bk; hist_rel[x] = 0.f; }
-        }
-        if constexpr (!KV)
-            for (int x = tid; x < p.n_buckets; x += kBwdThreads) hist[x] = 0.f;
-    }
-
     // own rows as B operands: lane (lr, hh) holds elements 16 s + 8 hh .. + 7 of its row
     const bool own_ok = own_row < n_own;
     v8 fa[KS], fb[KS];
@@ -534,6 +524,18 @@ __global__ __launch_bounds__(kBwdThreads, 2) void bwd16_kernel(const BwdParams p
     // Tile t + 1 is requested when the barrier at the top of tile t has shown that every wavefront is done with the
     // buffer it goes into, and has all of tile t's work to arrive in.
     if (t_lo < t_hi) { request(t_lo, 0); fetch_stat(t_lo); stage_stat(0); }
+    // the per-distance bias (and bucket) table, behind the first tile's requests and the loads of the own rows: its
+    // look-ups in the bias table are one more round trip to memory, which now runs beside theirs
+    if (has_bias) {
+        for (int x = tid; x <= 2 * sat; x += kBwdThreads) {
+            const int bk = bucket_of(p.bs, x - sat);
+            lut_bias[x] = load_table(p.table, p.table_dtype, (int64_t)bk * p.t_sbucket + (int64_t)h * p.t_shead) * 1.4426950408889634f;
+            if constexpr (!KV) { lut_bucket[x] = bk; hist_rel[x] = 0.f; }
+        }
+        if constexpr (!KV)
+            for (int x = tid; x < p.n_buckets; x += kBwdThreads) hist[x] = 0.f;
+    }
+
     for (int t = t_lo; t < t_hi; ++t) {
         const int o0 = t * kBwdOther;
         const int buf = (t - t_lo) & 1;
